@@ -1,0 +1,185 @@
+"""Benchmark of the two hot paths on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--path both|attn|lion] [--no-cpu-baseline]
+
+Prints ONE JSON line. The headline value is the attention forward throughput at B=2 H=16 S=8192 D=128 bf16 causal
+(FLOPs counted as 2*B*H*S^2*D); the fused Lion step over 1,308,622,848 fp32 parameters with bf16 momentum (16 bytes
+per parameter) is reported in the "lion" object of the same line, each with its roofline and a CPU baseline timed on
+this host's cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_MFMA_TFLOPS = 2500.0     # MI355X dense bf16/fp16
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
+
+def _events(n):
+    import torch
+
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def _time_steps(step, steps, warmup):
+    """W untimed steps, then K timed steps bracketed by synchronize; per-launch durations from HIP events recorded on
+    the stream the kernels are launched on (torch's current stream)."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = _events(steps + 1)
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        step()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per_launch = [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
+    return wall_ms / steps, sum(per_launch) / steps, min(per_launch)
+
+
+def bench_attention(steps, warmup, cpu_baseline):
+    import torch
+
+    from fast_ops.flash_attention.flash_attention import multi_head_attention
+
+    B, H, S, D = 2, 16, 8192, 128
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
+    scale = 1.0 / (D ** 0.5)
+    flops = 2.0 * B * H * S * S * D      # causal-halved 4*B*H*S^2*D
+    out = {}
+
+    def step():
+        out["o"], out["lse"] = multi_head_attention(q, k, v, causal=True, softmax_scale=scale, return_lse=True)
+
+    ms_step, ms_kernel, ms_min = _time_steps(step, steps, warmup)
+    res = {
+        "value": flops / (ms_step * 1e-3) / 1e12,
+        "ms_per_step": ms_step,
+        "roofline": {
+            "bound": "mfma", "achieved": flops / (ms_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+            "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": None,
+            "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "flops_per_launch": flops,
+        },
+        "workload": f"attention fwd B={B} H={H} S={S} D={D} bf16 causal, scale 1/sqrt({D})",
+    }
+    if cpu_baseline:
+        # bounded sample: ONE (batch, head) slice of the same shape through the oracle's fp32 vanilla path on all host cores
+        from oracle.attention_oracle import attention_fwd_oracle
+
+        torch.set_num_threads(os.cpu_count())
+        qs, ks, vs = (t[:1, :1].cpu() for t in (q, k, v))
+        attention_fwd_oracle(qs[:, :, :1024], ks[:, :, :1024], vs[:, :, :1024], causal=True, softmax_scale=scale)   # warm-up
+        t0 = time.perf_counter()
+        attention_fwd_oracle(qs, ks, vs, causal=True, softmax_scale=scale)
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {
+            "value": 2.0 * S * S * D / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 of {B * H} (batch, head) slices of the same shape, fp32 vanilla softmax(QK^T)V on the host, {dt:.2f} s",
+        }
+    return res
+
+
+def bench_lion(steps, warmup, cpu_baseline):
+    import torch
+
+    from fast_ops.lion.lion_optimizer import Lion
+
+    dev = "cuda:0"
+    shapes = [(2048, 8192)] * 39 + [(8192, 2048)] * 39
+    n_params = sum(a * b for a, b in shapes)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    params = [torch.nn.Parameter(torch.randn(s, device=dev, generator=gen) * 0.02) for s in shapes]
+    hp = dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
+    opt = Lion(params, **hp)
+    for p in params:
+        opt.state[p]["exp_avg"] = (torch.randn(p.shape, device=dev, generator=gen) * 1e-3).to(torch.bfloat16)
+        p.grad = torch.randn(p.shape, device=dev, generator=gen) * 1e-2
+    nbytes = 16.0 * n_params
+    ms_step, ms_kernel, ms_min = _time_steps(opt.step, steps, warmup)
+    res = {
+        "value": nbytes / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms_step, "dtype": "f32 params/grads, bf16 momentum",
+        "roofline": {
+            "bound": "hbm", "achieved": nbytes / (ms_kernel * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": nbytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+            "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "bytes_per_launch": nbytes,
+        },
+        "workload": f"fused Lion step, {len(shapes)} tensors (39 x 2048x8192 + 39 x 8192x2048) = {n_params} fp32 params, bf16 momentum",
+    }
+    if cpu_baseline:
+        # bounded sample: one 2048x8192 tensor (1/78 of the workload) through the four reference statements on all host cores
+        from oracle.lion_oracle import lion_step_torch
+
+        torch.set_num_threads(os.cpu_count())
+        p = params[0].detach().cpu().clone()
+        g = params[0].grad.cpu().clone()
+        m = opt.state[params[0]]["exp_avg"].cpu().clone()
+        lion_step_torch([p], [g], [m], hp["lr"], hp["betas"], hp["weight_decay"])     # warm-up
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            lion_step_torch([p], [g], [m], hp["lr"], hp["betas"], hp["weight_decay"])
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {
+            "value": 16.0 * p.numel() / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 of 78 tensors (2048x8192), vanilla 4-statement PyTorch Lion step on the host, {dt * 1e3:.1f} ms per step",
+        }
+    del opt, params
+    torch.cuda.empty_cache()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--path", choices=["both", "attn", "lion"], default="both")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: both kernels are single-device and this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from fast_ops_amd import _lib
+
+    _lib.load()   # fail loudly when the HIP library is missing
+    cpu = not args.no_cpu_baseline
+    attn = bench_attention(args.steps, args.warmup, cpu) if args.path in ("both", "attn") else None
+    lion = bench_lion(args.steps, args.warmup, cpu) if args.path in ("both", "lion") else None
+    head = attn if attn is not None else lion
+    line = {
+        "metric": "FA fwd TFLOP/s (bf16, S=8K D=128 causal) + fused Lion HBM GB/s",
+        "value": head["value"],
+        "unit": "TFLOP/s" if attn is not None else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if attn is not None else "f32",
+        "data": "synthetic",
+        "config": {"workload": head["workload"] + ("; second path: " + lion["workload"] if attn is not None and lion is not None else "")},
+        "roofline": head["roofline"],
+    }
+    if "cpu_baseline" in head:
+        line["cpu_baseline"] = head["cpu_baseline"]
+    if attn is not None and lion is not None:
+        line["lion"] = {k: v for k, v in lion.items() if k != "workload"}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

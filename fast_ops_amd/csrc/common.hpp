@@ -1,0 +1,27 @@
+// Shared helpers for the HIP sources of libfastops_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fastops.h"
+
+namespace fo {
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) uint16_t u16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
+// variant selectors set through fo_tune_set (-1 = default)
+extern int g_lion_variant;
+extern int g_attn_variant;
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? FO_OK : FO_ERR_LAUNCH; }
+
+}  // namespace fo

@@ -1,0 +1,170 @@
+"""Fused Lion optimizer for MI355X: drop-in for ``fast_ops.lion.lion_optimizer.Lion``.
+
+Same constructor, validation, state key and ``step()`` semantics as the reference class
+(fast_ops/lion/lion_optimizer.py:29-76); the arithmetic is that of the reference formula
+(fast_ops/lion/lion_optimizer_ref.py:51,64,65,67) for fp32 parameters and gradients with a bf16 momentum.
+
+What differs from the reference, on purpose:
+
+* one kernel launch per parameter group instead of one per parameter (lion_optimizer.py:64-76 launches per tensor):
+  the tensors of a group are cut into 8192-element chunks whose descriptors live in a device table that is rebuilt
+  only when a parameter, gradient or momentum pointer changes;
+* parameters and gradients are fp32 and the momentum is bf16 (the reference kernel requires one half dtype for all
+  three, lion_update.cu:132-135); the momentum dtype for freshly created state is ``exp_avg_dtype``;
+* the six scalar constants are computed here in Python double precision and rounded once to fp32, which is what the
+  reference formula's Python expressions do.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Iterable, List, Optional, Tuple
+
+import numpy as np
+import torch
+from torch import Tensor
+from torch.nn import Parameter
+from torch.optim.optimizer import Optimizer
+
+from .. import _lib
+
+_CHUNK_DTYPE = np.dtype([("p", "<u8"), ("g", "<u8"), ("m", "<u8"), ("n", "<i4"), ("reserved", "<i4")])
+assert _CHUNK_DTYPE.itemsize == ctypes.sizeof(_lib.FoLionChunk) == 32
+
+
+def _dense_same_layout(a: Tensor, *others: Tensor) -> bool:
+    """True when `a` is non-overlapping and dense and the others share its strides exactly (element i of one is
+    element i of the others in memory order). The reference checks density only (lion_update.cu:109-112,137-139)."""
+    if any(o.shape != a.shape or o.stride() != a.stride() for o in others):
+        return False
+    if a.is_contiguous():
+        return True
+    expect = 1
+    for size, stride in sorted(((s, st) for s, st in zip(a.shape, a.stride()) if s != 1), key=lambda x: x[1]):
+        if stride != expect:
+            return False
+        expect *= size
+    return True
+
+
+def make_consts(lr: float, betas: Tuple[float, float], weight_decay: float) -> "_lib.FoLionConsts":
+    c = _lib.FoLionConsts()
+    _lib.check(_lib.load().fo_lion_make_consts(float(lr), float(betas[0]), float(betas[1]), float(weight_decay), ctypes.byref(c)),
+               "fo_lion_make_consts")
+    return c
+
+
+def build_chunk_table(ptrs: List[Tuple[int, int, int, int]]) -> np.ndarray:
+    """(p_ptr, g_ptr, m_ptr, numel) per tensor -> structured array of fo_lion_chunk descriptors."""
+    C = _lib.FO_LION_CHUNK
+    parts = []
+    for p_ptr, g_ptr, m_ptr, numel in ptrs:
+        if numel == 0:
+            continue
+        n = (numel + C - 1) // C
+        off = np.arange(n, dtype=np.uint64) * np.uint64(C)
+        t = np.zeros(n, dtype=_CHUNK_DTYPE)
+        t["p"] = np.uint64(p_ptr) + off * np.uint64(4)
+        t["g"] = np.uint64(g_ptr) + off * np.uint64(4)
+        t["m"] = np.uint64(m_ptr) + off * np.uint64(2)
+        t["n"] = np.minimum(np.uint64(C), np.uint64(numel) - off).astype(np.int32)
+        parts.append(t)
+    return np.concatenate(parts) if parts else np.zeros(0, dtype=_CHUNK_DTYPE)
+
+
+def lion_update(param: Tensor, grad: Tensor, exp_avg: Tensor, lr: float, beta1: float, beta2: float, weight_decay: float) -> None:
+    """Single-tensor in-place update: the call the reference extension exposes (fast_ops/lion/lion.cpp:4-15)."""
+    _check_tensors(param, grad, exp_avg)
+    c = make_consts(lr, (beta1, beta2), weight_decay)
+    with torch.cuda.device(param.device):
+        stream = torch.cuda.current_stream(param.device).cuda_stream
+        _lib.check(
+            _lib.load().fo_lion_update(param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), param.numel(), ctypes.byref(c), stream),
+            "fo_lion_update",
+        )
+
+
+def _check_tensors(param: Tensor, grad: Tensor, exp_avg: Tensor) -> None:
+    if not (param.is_cuda and grad.is_cuda and exp_avg.is_cuda):
+        raise RuntimeError("fused Lion runs on the GPU only: parameters, gradients and momentum must be device tensors")
+    if not (param.device == grad.device == exp_avg.device):
+        raise RuntimeError("parameter, gradient and momentum must live on the same device")
+    if param.dtype != torch.float32 or grad.dtype != torch.float32 or exp_avg.dtype != torch.bfloat16:
+        raise RuntimeError(
+            f"unsupported dtypes (param {param.dtype}, grad {grad.dtype}, exp_avg {exp_avg.dtype}): "
+            "this kernel takes float32 parameters and gradients with a bfloat16 momentum"
+        )
+    if grad.is_sparse:
+        raise RuntimeError("Lion does not support sparse gradients")
+    if not _dense_same_layout(param, grad, exp_avg):
+        raise RuntimeError("expected tensor to be contiguous")   # message of lion_update.cu:109-112
+
+
+class Lion(Optimizer):
+    """Lion optimizer ("Symbolic Discovery of Optimization Algorithms", https://arxiv.org/abs/2302.06675), fused."""
+
+    def __init__(
+        self,
+        params: Iterable[Parameter],
+        lr: float = 1e-4,
+        betas: Tuple[float, float] = (0.9, 0.99),
+        weight_decay: float = 0.0,
+        *,
+        exp_avg_dtype: torch.dtype = torch.bfloat16,
+    ) -> None:
+        """
+        :param params: iterable of parameters to optimize or dicts defining parameter groups
+        :param lr: learning rate
+        :param betas: coefficients of the update interpolation and of the momentum decay
+        :param weight_decay: decoupled weight decay coefficient
+        :param exp_avg_dtype: dtype of momentum buffers this optimizer creates (state loaded or seeded by the caller
+          keeps its own dtype)
+        """
+        # same checks, exception type and messages as lion_optimizer.py:49-52
+        if lr <= 0:
+            raise RuntimeError(f"expected positive LR, got {lr}")
+        if not all(0 <= beta <= 1 for beta in betas):
+            raise RuntimeError(f"betas must be between 0 and 1. got {betas}")
+        if exp_avg_dtype != torch.bfloat16:
+            raise RuntimeError(f"exp_avg_dtype {exp_avg_dtype} is not implemented: the fused kernel keeps a bfloat16 momentum")
+        defaults = {"lr": lr, "betas": betas, "weight_decay": weight_decay}
+        super().__init__(params, defaults)
+        self._exp_avg_dtype = exp_avg_dtype
+        # (group index, device) -> (key of data pointers, device table tensor, number of chunks)
+        self._tables: Dict[Tuple[int, torch.device], Tuple[tuple, Tensor, int]] = {}
+        _lib.load()   # fail at construction, not at the first step, when the library is missing
+
+    @torch.no_grad()
+    def step(self) -> None:
+        """Parameter and state (momentum) update: one fused launch per parameter group and device."""
+        lib = _lib.load()
+        for gi, group in enumerate(self.param_groups):
+            lr = group["lr"]
+            weight_decay = group["weight_decay"]
+            beta1, beta2 = group["betas"]
+            per_device: Dict[torch.device, List[Tuple[int, int, int, int]]] = {}
+            for param in group["params"]:
+                grad: Optional[Tensor] = param.grad
+                if grad is None:
+                    continue
+                state = self.state[param]
+                if "exp_avg" not in state:
+                    # exponential moving average of the gradient (lion_optimizer.py:68-73), kept in bf16
+                    state["exp_avg"] = torch.zeros_like(param, dtype=self._exp_avg_dtype, memory_format=torch.preserve_format)
+                exp_avg: Tensor = state["exp_avg"]
+                _check_tensors(param, grad, exp_avg)
+                per_device.setdefault(param.device, []).append((param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), param.numel()))
+            if not per_device:
+                continue
+            consts = make_consts(lr, (beta1, beta2), weight_decay)
+            for device, ptrs in per_device.items():
+                key = tuple(ptrs)
+                cached = self._tables.get((gi, device))
+                if cached is None or cached[0] != key:
+                    table = build_chunk_table(ptrs)
+                    table_dev = torch.from_numpy(table.view(np.uint8)).to(device)
+                    cached = (key, table_dev, int(table.shape[0]))
+                    self._tables[(gi, device)] = cached
+                _, table_dev, n_chunks = cached
+                with torch.cuda.device(device):
+                    stream = torch.cuda.current_stream(device).cuda_stream
+                    _lib.check(lib.fo_lion_step(table_dev.data_ptr(), n_chunks, ctypes.byref(consts), stream), "fo_lion_step")

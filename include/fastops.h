@@ -1,0 +1,128 @@
+/* fastops.h - C ABI of libfastops_hip.so: FlashAttention forward and the fused Lion step for AMD MI355X (gfx950).
+ *
+ * This is the boundary that replaces the reference's two pybind11 torch extensions:
+ *   fast_ops/flash_attention/flash_attention.cpp:12-14   forward(Q, K, V) -> O
+ *   fast_ops/lion/lion.cpp:13-15                         lion_update(param, grad, exp_avg, lr, beta1, beta2, wd)
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every pointer is a device pointer unless its name ends in _host;
+ *   - the library allocates nothing, frees nothing and keeps no pointer after a call returns;
+ *   - every call is asynchronous on the hipStream_t passed as `stream` (NULL = the default stream), never
+ *     synchronises, and may be issued from several host threads on different streams;
+ *   - return value 0 (FO_OK) or a negative fo_status; nothing throws or aborts. All argument checks happen before
+ *     any HIP call, so a rejected call has touched neither the device nor the stream.
+ */
+#ifndef FASTOPS_H_
+#define FASTOPS_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum fo_status {
+  FO_OK = 0,
+  FO_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+  FO_ERR_BAD_DTYPE = -2,      /* dtype code is not FO_DTYPE_F16 / FO_DTYPE_BF16 (the reference dispatches half types only,
+                                 flash_attention/common/launch_utils.h:8-21) */
+  FO_ERR_BAD_HEAD_DIM = -3,   /* head_dim not supported (reference contract: <= 128 and a multiple of 8,
+                                 flash_attention.py:61-66; this library implements 64 and 128) */
+  FO_ERR_BAD_SHAPE = -4,      /* a size is <= 0, or too large for the kernel's indexing */
+  FO_ERR_BAD_STRIDE = -5,     /* a stride breaks the layout contract (rows must be 16-byte aligned) */
+  FO_ERR_MISALIGNED = -6,     /* a base pointer is not aligned as required */
+  FO_ERR_LAUNCH = -7,         /* hipGetLastError() reported a failure after the launch (the reference's
+                                 C10_CUDA_KERNEL_LAUNCH_CHECK, lion_update.cu:159) */
+  FO_ERR_UNSUPPORTED = -8     /* valid request that this build does not implement */
+} fo_status;
+
+enum { FO_DTYPE_F16 = 0, FO_DTYPE_BF16 = 1 };
+
+/* Human-readable text for a status code; never NULL. */
+const char* fo_strerror(int status);
+
+/* Library ABI version: major*1000 + minor. */
+int fo_version(void);
+
+/* Tuning hook for benchmarks and profiling: selects a kernel variant by name ("lion.variant", "attn.variant").
+ * The defaults are the measured best; value -1 restores the default. Returns FO_OK or FO_ERR_UNSUPPORTED for an
+ * unknown key or value. Process-global and not synchronised with calls in flight. No reference counterpart. */
+int fo_tune_set(const char* key, int value);
+int fo_tune_get(const char* key);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * FlashAttention forward.
+ * Replaces flash_attn_fwd / flash_attn_fwd_cuda (flash_attention.cpp:5-10, flash_attention_fwd.cu:154-181) and
+ * implements what that unfinished kernel's comments describe (flash_attention_fwd.cu:37-47,120-151) with the numerics
+ * of the reference's working Triton forward (flash_attention_triton.py:128-255): O = softmax(scale * Q K^T + mask) V
+ * with fp32 scores and accumulators, and LSE = natural-log logsumexp of the scaled, masked scores.
+ *
+ *   q            [B, H, Sq, D]   element (b,h,s,d) at q + b*q_strides[0] + h*q_strides[1] + s*q_strides[2] + d
+ *   k, v         [B, H, Sk, D]   same addressing with their own strides
+ *   o            [B, H, Sq, D]   written for every (b,h,s,d); never read
+ *   lse          [B, H, Sq] fp32, contiguous; may be NULL when the caller does not want it
+ *   *_strides    three element strides (batch, head, sequence); the head_dim stride is 1. A [B,S,H,D] tensor (the
+ *                layout of flash_attention_triton.py:734-737) is passed by swapping the head and sequence strides;
+ *                a head stride of 0 expresses multi-query K/V.
+ *   causal       non-zero: query i attends keys j <= i (top-left aligned, attention_ref.py:54-58)
+ *   dtype        FO_DTYPE_F16 or FO_DTYPE_BF16, for q, k, v and o alike
+ *
+ * Requirements checked here: D in {64, 128}; Sq, Sk >= 1; base pointers and row strides multiples of 16 bytes.
+ */
+int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                int B, int H, int Sq, int Sk, int D,
+                const int64_t* q_strides_host, const int64_t* k_strides_host,
+                const int64_t* v_strides_host, const int64_t* o_strides_host,
+                float softmax_scale, int causal, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * Fused Lion step: fp32 parameters, fp32 gradients, bf16 momentum, one pass.
+ * Per element, in this order and with these rounding points (lion_optimizer_ref.py:51,64,65,67):
+ *     p1 = p * c_wd
+ *     u  = f32(bf16(m * c_b1)) + g * c_1b1
+ *     p  = p1 + c_nlr * sign(u)                 sign(+-0) = sign(NaN) = 0
+ *     m  = bf16( fma(c_1b2, g, f32(bf16(m * c_b2))) )
+ * bf16() is round-to-nearest-even (NaN -> 0x7FC0). The kernel fuses what lion_update_kernel fuses
+ * (lion_update.cu:44-106) but keeps the fp32 rounding points of the Python formula instead of half arithmetic.
+ */
+typedef struct fo_lion_consts {
+  float c_wd;   /* f32(1 - lr*weight_decay) */
+  float c_b1;   /* f32(beta1)               */
+  float c_1b1;  /* f32(1 - beta1)           */
+  float c_nlr;  /* f32(-lr)                 */
+  float c_b2;   /* f32(beta2)               */
+  float c_1b2;  /* f32(1 - beta2)           */
+} fo_lion_consts;
+
+/* Computes the six constants in double precision and rounds each once to fp32, exactly as the Python expressions of
+ * lion_optimizer_ref.py:51,64,65,67 do. Host-only; `out_host` is host memory. */
+int fo_lion_make_consts(double lr, double beta1, double beta2, double weight_decay, fo_lion_consts* out_host);
+
+/* One tensor, in place. Replaces lion_update (lion.cpp:4-15, lion_update.cu:121-161). Any numel >= 0 and any
+ * alignment of 4 bytes (p, g) / 2 bytes (m) is accepted; 16-byte aligned p, g and 8-byte aligned m take the
+ * vector path. */
+int fo_lion_update(float* p, const float* g, uint16_t* m, int64_t numel, const fo_lion_consts* consts_host, void* stream);
+
+/* Many tensors in one launch. Replaces the per-parameter loop of Lion.step (lion_optimizer.py:64-76).
+ * The caller splits every tensor into chunks of at most FO_LION_CHUNK elements (all but a tensor's last chunk are
+ * exactly FO_LION_CHUNK long) and passes, in device memory, one descriptor per chunk. */
+#define FO_LION_CHUNK 8192
+
+typedef struct fo_lion_chunk {
+  float* p;          /* first parameter of the chunk                          */
+  const float* g;    /* first gradient of the chunk                           */
+  uint16_t* m;       /* first momentum element (bf16 bit pattern) of the chunk */
+  int32_t n;         /* elements in this chunk, 1..FO_LION_CHUNK              */
+  int32_t reserved;  /* must be 0                                             */
+} fo_lion_chunk;
+
+int fo_lion_step(const fo_lion_chunk* chunks_dev, int64_t n_chunks, const fo_lion_consts* consts_host, void* stream);
+
+/* Host-only helper: fills `out_host[0 .. return value)` with the chunk descriptors of one tensor and returns how many
+ * it wrote (ceil(numel / FO_LION_CHUNK)); with out_host == NULL it only counts. */
+int64_t fo_lion_fill_chunks(float* p, const float* g, uint16_t* m, int64_t numel, fo_lion_chunk* out_host);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTOPS_H_ */

@@ -1,0 +1,102 @@
+"""CPU oracle for the attention forward pass (TEST INFRASTRUCTURE ONLY - never imported by the product).
+
+Restates, with torch CPU ops in fp32, what the reference defines:
+
+* output: ``fast_ops/flash_attention/attention_ref.py:41-49,54-59,67`` - upcast q/k/v to fp32, scores =
+  (q * scale) . k^T, causal mask = strict upper triangle (top-left aligned) set to -inf, softmax over keys, times v.
+  The reference divides q by sqrt(d); the Triton surface takes an arbitrary ``softmax_scale``
+  (``flash_attention_triton.py:750``), so the scale is a parameter here and defaults to 1/sqrt(d).
+* logsumexp: ``fast_ops/flash_attention/flash_attention_triton.py:201-203,241-243,255`` - natural-log
+  logsumexp of the *scaled* scores over the unmasked keys, one fp32 value per query row.
+* the tile recurrence itself (``flash_attention_triton.py:128-129,149,169-175,200-213,237-250``) is restated in
+  ``online_softmax_tiles`` so that tests can show recurrence == closed form, including the running reference
+  being ``lse_i`` rather than ``m_i``.
+
+Layout is the drop-in surface's: Q [B,H,M,D], K/V [B,H,N,D] (``flash_attention.py:30-37``).
+
+Pinned by tests/test_oracle_attention.py against: torch.nn.functional.scaled_dot_product_attention (independent
+library routine), torch.logsumexp, a float64 triple-loop brute force on tiny inputs, and closed-form invariants
+(V == 1, Q == 0, causal row 0, key permutation, one-hot selection).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+
+def attention_fwd_oracle(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    causal: bool = False,
+    softmax_scale: Optional[float] = None,
+    q_chunk: int = 1024,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 softmax(scale * Q K^T + mask) V and its logsumexp. Returns (O fp32 [B,H,M,D], LSE fp32 [B,H,M]).
+
+    Works one (batch, head) slice and ``q_chunk`` query rows at a time so that S = 8192 does not materialise
+    the full [B,H,M,N] score tensor (attention_ref.py does; same arithmetic per row).
+    """
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    qf, kf, vf = q.float().cpu(), k.float().cpu(), v.float().cpu()   # attention_ref.py:41-43
+    out = torch.empty(B, H, M, D, dtype=torch.float32)
+    lse = torch.empty(B, H, M, dtype=torch.float32)
+    for b in range(B):
+        for h in range(H):
+            kt = kf[b, h].t()
+            for m0 in range(0, M, q_chunk):
+                m1 = min(M, m0 + q_chunk)
+                scores = (qf[b, h, m0:m1] * scale) @ kt                      # attention_ref.py:46-47
+                if causal:
+                    rows = torch.arange(m0, m1).unsqueeze(1)
+                    cols = torch.arange(N).unsqueeze(0)
+                    scores = scores.masked_fill(cols > rows, float("-inf"))  # attention_ref.py:54-58 (triu, diagonal=1)
+                lse[b, h, m0:m1] = torch.logsumexp(scores, dim=-1)
+                attn = torch.softmax(scores, dim=-1)                          # attention_ref.py:59
+                out[b, h, m0:m1] = attn @ vf[b, h]                            # attention_ref.py:67
+    return out, lse
+
+
+def online_softmax_tiles(
+    q: np.ndarray, k: np.ndarray, v: np.ndarray, causal: bool, scale: float, block_m: int = 128, block_n: int = 128
+) -> Tuple[np.ndarray, np.ndarray]:
+    """The reference's tile recurrence for one (batch, head): q [M,D], k/v [N,D] float32 -> (O [M,D], LSE [M]).
+
+    Follows flash_attention_triton.py: state init :128-130, causal loop bound :149, qk :169-170, causal -inf :174-175,
+    m_ij / p / l_ij :200-203, accumulator rescale :206-213, PV :237-238, state update :241-243, epilogue :245-250,255.
+    P is *not* rounded to half here (this function pins the recurrence, not the operand rounding).
+    """
+    M, D = q.shape
+    N = k.shape[0]
+    out = np.zeros((M, D), np.float32)
+    lse_out = np.zeros((M,), np.float32)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        for start_m in range(0, M, block_m):
+            rows = np.arange(start_m, min(M, start_m + block_m))
+            qi = q[rows]
+            lse_i = np.full(len(rows), -np.inf, np.float32)
+            m_i = np.full(len(rows), -np.inf, np.float32)
+            acc = np.zeros((len(rows), D), np.float32)
+            end_n = N if not causal else min(start_m + block_m, N)
+            for start_n in range(0, end_n, block_n):
+                cols = np.arange(start_n, min(N, start_n + block_n))
+                qk = (qi @ k[cols].T).astype(np.float32)
+                if causal:
+                    qk = qk + np.where(rows[:, None] >= cols[None, :], 0.0, -np.inf).astype(np.float32)
+                m_ij = np.maximum(qk.max(axis=1) * np.float32(scale), lse_i)
+                p = np.exp(qk * np.float32(scale) - m_ij[:, None]).astype(np.float32)
+                l_ij = p.sum(axis=1, dtype=np.float32)
+                acc = acc * np.exp(m_i - m_ij)[:, None]
+                acc = acc + p @ v[cols]
+                m_i = m_ij
+                lse_i = (m_ij + np.log(np.exp(lse_i - m_ij) + l_ij)).astype(np.float32)
+            acc = acc * np.exp(m_i - lse_i)[:, None]
+            out[rows] = acc
+            lse_out[rows] = lse_i
+    return out, lse_out

@@ -1,0 +1,177 @@
+"""Parity of the attention forward kernel (through the C ABI) with the CPU oracle.
+
+Tolerances are the ones the task states: O within atol 2e-2 / rtol 1e-2 of fp32 softmax(scale Q K^T) V computed
+from the same half-precision inputs, LSE within 1e-3 (absolute). Inputs are drawn on the CPU from a seeded
+generator in fp32, rounded to the operand type, then copied, so both sides see identical bits."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from fast_ops.flash_attention.flash_attention import FlashAttentionFunction, flash_attn, multi_head_attention
+from oracle.attention_oracle import attention_fwd_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+O_ATOL, O_RTOL, LSE_ATOL = 2e-2, 1e-2, 1e-3
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "attn_small.npz")
+
+
+def _qkv(B, H, Sq, Sk, D, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    k = torch.randn(B, H, Sk, D, generator=g).to(dtype)
+    v = torch.randn(B, H, Sk, D, generator=g).to(dtype)
+    return q, k, v
+
+
+def _check(o, lse, o_ref, lse_ref, what=""):
+    o = o.float().cpu()
+    lse = lse.cpu()
+    err = (o - o_ref).abs()
+    bound = O_ATOL + O_RTOL * o_ref.abs()
+    worst = float((err - bound).max())
+    assert worst <= 0, f"{what}: O outside atol {O_ATOL} / rtol {O_RTOL} by {worst:.3e} (max abs err {float(err.max()):.3e})"
+    lse_err = float((lse - lse_ref).abs().max())
+    assert lse_err <= LSE_ATOL, f"{what}: LSE error {lse_err:.3e} > {LSE_ATOL}"
+    return float(err.max()), lse_err
+
+
+def _run_and_check(B, H, Sq, Sk, D, dtype, causal, seed=0, scale=None):
+    q, k, v = _qkv(B, H, Sq, Sk, D, dtype, seed)
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, softmax_scale=scale)
+    o, lse = multi_head_attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal, softmax_scale=scale, return_lse=True)
+    torch.cuda.synchronize()
+    assert o.dtype == dtype and o.shape == q.shape and lse.dtype == torch.float32 and lse.shape == (B, H, Sq)
+    return _check(o, lse, o_ref, lse_ref, f"B{B} H{H} Sq{Sq} Sk{Sk} D{D} {dtype} causal={causal}")
+
+
+def test_config1_tiny_fp16_noncausal():
+    # B=2 H=4 S=128 D=64, fp16, non-causal, scale 1/8
+    _run_and_check(2, 4, 128, 128, 64, torch.float16, False, seed=0, scale=0.125)
+
+
+def test_config2_gpt2_small_bf16_causal():
+    # B=8 H=12 S=1024 D=64, bf16, causal, scale 1/8
+    _run_and_check(8, 12, 1024, 1024, 64, torch.bfloat16, True, seed=0, scale=0.125)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_dtype_causal_headdim_grid(dtype, causal, D):
+    _run_and_check(2, 3, 512, 512, D, dtype, causal, seed=3)
+
+
+def test_long_context_slice_of_headline_shape():
+    # the headline shape is B=2 H=16 S=8192 D=128 bf16 causal; two of its (batch, head) slices against the oracle
+    _run_and_check(1, 2, 8192, 8192, 128, torch.bfloat16, True, seed=0)
+
+
+def test_throughput_shape_slice_fp16_noncausal():
+    # B=16 H=32 S=2048 D=128 fp16 non-causal; 8 of its (batch, head) slices
+    _run_and_check(1, 8, 2048, 2048, 128, torch.float16, False, seed=0)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 1000), (1, 1, 1000, 64), (3, 5, 191, 191)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_ragged_and_unequal_lengths(shape, causal, D):
+    # sequence lengths that are not multiples of the 128-row / 64-key tiles, Sq != Sk (causal mask is top-left aligned)
+    B, H, Sq, Sk = shape
+    _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
+
+
+def test_golden_fixture():
+    z = np.load(GOLDEN)
+    to16 = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16)
+    q, k, v = (to16(z[n]).to(DEV) for n in "qkv")
+    for tag, causal in (("full", False), ("causal", True)):
+        o, lse = multi_head_attention(q, k, v, causal=causal, softmax_scale=float(z["scale"]), return_lse=True)
+        _check(o, lse, torch.from_numpy(z[f"o_{tag}"]), torch.from_numpy(z[f"lse_{tag}"]), f"golden {tag}")
+
+
+def test_bshd_surface_and_multi_query():
+    # [batch, seqlen, nheads, headdim] inputs (flash_attention_triton.py:734-737); K/V shared across heads via expand,
+    # as tests/test_flash_attention_triton.py:71-73 does
+    B, S, H, D = 2, 300, 4, 128
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16)
+    kv = torch.randn(B, S, 2, 1, D, generator=g).to(torch.bfloat16)
+    k, v = kv.unbind(2)
+    k, v = k.expand(B, S, H, D), v.expand(B, S, H, D)
+    o_ref, lse_ref = attention_fwd_oracle(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), causal=True)
+    qd = q.to(DEV)
+    kd, vd = (t.to(DEV).expand(B, S, H, D) for t in kv.unbind(2))
+    o, lse = flash_attn(qd, kd, vd, causal=True, return_lse=True)
+    assert o.shape == (B, S, H, D)
+    _check(o.transpose(1, 2), lse, o_ref, lse_ref, "BSHD multi-query")
+    with pytest.raises(RuntimeError, match="bias"):
+        flash_attn(qd, kd, vd, bias=torch.zeros(1, device=DEV))
+    with pytest.raises(RuntimeError, match="dropout"):
+        flash_attn(qd, kd, vd, dropout_p=0.1)
+
+
+def test_non_contiguous_head_slices():
+    # Q/K/V as slices of one packed [B, S, 3, H, D] projection output
+    B, S, H, D = 1, 256, 2, 64
+    g = torch.Generator().manual_seed(6)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).to(torch.float16)
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))   # [B, H, S, D] views, not contiguous
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=False)
+    qd = qkv.to(DEV)
+    o, lse = multi_head_attention(*(qd[:, :, i].permute(0, 2, 1, 3) for i in range(3)), return_lse=True)
+    _check(o, lse, o_ref, lse_ref, "packed qkv views")
+
+
+def test_closed_form_invariants_at_full_headline_size():
+    """B=2 H=16 S=8192 D=128 bf16 causal (the benchmark shape): properties that need no oracle.
+    V == 1 => O == 1 exactly; Q == 0 => LSE_i = ln(i+1) and O_i = running mean of V; the last causal row equals the
+    non-causal result for that row; two runs give identical bits."""
+    B, H, S, D = 2, 16, 8192, 128
+    g = torch.Generator(device=DEV).manual_seed(0)
+    q = torch.randn(B, H, S, D, device=DEV, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, H, S, D, device=DEV, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, H, S, D, device=DEV, generator=g).to(torch.bfloat16)
+    o1, lse1 = multi_head_attention(q, k, v, causal=True, return_lse=True)
+    o2, lse2 = multi_head_attention(q, k, v, causal=True, return_lse=True)
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2), "kernel is not deterministic"
+    assert bool(torch.isfinite(o1.float()).all()) and bool(torch.isfinite(lse1).all())
+    o_ones = multi_head_attention(q, k, torch.ones_like(v), causal=True)
+    assert float((o_ones.float() - 1).abs().max()) <= 2 ** -7          # sum of bf16-rounded weights / fp32 sum
+    oz, lsez = multi_head_attention(torch.zeros_like(q), k, v, causal=True, return_lse=True)
+    want = torch.log(torch.arange(1, S + 1, device=DEV, dtype=torch.float32)).expand(B, H, S)
+    assert float((lsez - want).abs().max()) <= 1e-4
+    mean = torch.cumsum(v.float(), dim=2) / torch.arange(1, S + 1, device=DEV).view(1, 1, S, 1)
+    assert float((oz.float() - mean).abs().max()) <= 2e-2
+    o_nc, lse_nc = multi_head_attention(q[:, :, -128:], k, v, causal=False, return_lse=True)
+    assert float((o_nc[:, :, -1].float() - o1[:, :, -1].float()).abs().max()) <= 2e-2
+    assert float((lse_nc[:, :, -1] - lse1[:, :, -1]).abs().max()) <= 1e-3
+    # row 0 attends key 0 only
+    assert torch.equal(o1[:, :, 0], v[:, :, 0])
+
+
+def test_autograd_function_surface():
+    q, k, v = (t.to(DEV) for t in _qkv(1, 1, 128, 128, 64, torch.bfloat16, seed=9))
+    q.requires_grad_(True)
+    o = FlashAttentionFunction.apply(q, k, v)
+    assert o.requires_grad
+    with pytest.raises(NotImplementedError):
+        o.sum().backward()
+
+
+def test_rejected_inputs_raise():
+    q, k, v = (t.to(DEV) for t in _qkv(1, 1, 16, 16, 72, torch.bfloat16))
+    with pytest.raises(RuntimeError, match="head_dim"):
+        multi_head_attention(q, k, v)
+    q, k, v = (t.to(DEV) for t in _qkv(1, 1, 16, 16, 256, torch.bfloat16))
+    with pytest.raises(RuntimeError, match="up to 128"):
+        multi_head_attention(q, k, v)
+    q, k, v = (t.to(DEV) for t in _qkv(1, 1, 16, 16, 64, torch.float32))
+    with pytest.raises(RuntimeError, match="half-precision"):
+        multi_head_attention(q, k, v)
+    q, k, v = (t.to(DEV) for t in _qkv(1, 2, 16, 16, 64, torch.bfloat16))
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        multi_head_attention(q, k[:, :1], v)

@@ -1,0 +1,138 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol include/fastops.h declares, rejects bad
+arguments with the documented codes before touching a device, and its host-only helpers agree with the oracle."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from fast_ops_amd import _lib
+from fast_ops_amd.lion import lion_optimizer as lo_host
+from oracle import lion_oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fastops.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fo_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert set(declared) == set(_lib.SIGNATURES), "ctypes signature table and header disagree"
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/fastops.h but not exported"
+
+
+def test_version_and_strerror():
+    lib = _lib.load()
+    assert lib.fo_version() >= 1000
+    assert _lib.strerror(0) == "ok"
+    for code in range(-8, 0):
+        assert "unknown" not in _lib.strerror(code)
+    assert "unknown" in _lib.strerror(-99)
+
+
+def test_struct_layouts_match_header():
+    assert ctypes.sizeof(_lib.FoLionConsts) == 24
+    assert ctypes.sizeof(_lib.FoLionChunk) == 32
+    assert _lib.FoLionChunk.n.offset == 24
+    m = re.search(r"#define\s+FO_LION_CHUNK\s+(\d+)", open(HEADER).read())
+    assert int(m.group(1)) == _lib.FO_LION_CHUNK
+
+
+def test_attn_argument_validation_without_device():
+    lib = _lib.load()
+    s = (ctypes.c_int64 * 3)(128 * 64, 64 * 128 * 4, 64)   # dummy but well-formed strides
+    ok_ptr = 0x1000
+    call = lambda **kw: lib.fo_attn_fwd(
+        kw.get("q", ok_ptr), kw.get("k", ok_ptr), kw.get("v", ok_ptr), kw.get("o", ok_ptr), kw.get("lse", None),
+        kw.get("B", 1), kw.get("H", 1), kw.get("Sq", 128), kw.get("Sk", 128), kw.get("D", 64),
+        kw.get("qs", s), kw.get("ks", s), kw.get("vs", s), kw.get("os", s),
+        kw.get("scale", 0.125), 0, kw.get("dtype", 1), None)
+    assert call(q=None) == -1
+    assert call(qs=None) == -1
+    assert call(dtype=2) == -2
+    assert call(D=72) == -3
+    assert call(D=256) == -3
+    assert call(Sq=0) == -4
+    assert call(B=-1) == -4
+    bad = (ctypes.c_int64 * 3)(128 * 64, 64 * 128, 60)
+    assert call(ks=bad) == -5
+    assert call(q=0x1008) == -6
+    assert call(scale=float("nan")) == -4
+
+
+def test_lion_argument_validation_without_device():
+    lib = _lib.load()
+    c = _lib.FoLionConsts()
+    assert lib.fo_lion_make_consts(1e-4, 0.9, 0.99, 0.1, None) == -1
+    assert lib.fo_lion_update(0x1000, 0x1000, 0x1000, 16, None, None) == -1
+    assert lib.fo_lion_update(None, 0x1000, 0x1000, 16, ctypes.byref(c), None) == -1
+    assert lib.fo_lion_update(0x1000, 0x1000, 0x1000, -1, ctypes.byref(c), None) == -4
+    assert lib.fo_lion_update(0x1002, 0x1000, 0x1000, 16, ctypes.byref(c), None) == -6
+    assert lib.fo_lion_update(None, None, None, 0, ctypes.byref(c), None) == 0      # empty tensor: nothing to do
+    assert lib.fo_lion_step(None, 0, ctypes.byref(c), None) == 0
+    assert lib.fo_lion_step(None, 4, ctypes.byref(c), None) == -1
+    assert lib.fo_lion_step(0x1000, -1, ctypes.byref(c), None) == -4
+    assert lib.fo_lion_step(0x1004, 4, ctypes.byref(c), None) == -6
+
+
+@pytest.mark.parametrize("hp", [(1e-4, 0.9, 0.99, 0.1), (1e-3, 0.95, 0.98, 0.5), (3e-5, 0.0, 1.0, 0.0)])
+def test_make_consts_matches_python_double_arithmetic(hp):
+    lr, b1, b2, wd = hp
+    c = lo_host.make_consts(lr, (b1, b2), wd)
+    got = np.array([c.c_wd, c.c_b1, c.c_1b1, c.c_nlr, c.c_b2, c.c_1b2], dtype=np.float32)
+    want = np.array(lion_oracle.lion_consts(lr, (b1, b2), wd), dtype=np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_fill_chunks_matches_python_table():
+    lib = _lib.load()
+    for numel in (1, 8191, 8192, 8193, 50257 * 768):
+        n = lib.fo_lion_fill_chunks(0x10000000, 0x20000000, 0x30000000, numel, None)
+        assert n == -(-numel // _lib.FO_LION_CHUNK)
+        buf = (_lib.FoLionChunk * n)()
+        assert lib.fo_lion_fill_chunks(0x10000000, 0x20000000, 0x30000000, numel, buf) == n
+        table = lo_host.build_chunk_table([(0x10000000, 0x20000000, 0x30000000, numel)])
+        mine = np.frombuffer(buf, dtype=table.dtype)
+        assert np.array_equal(mine, table)
+        assert int(table["n"].sum()) == numel
+    assert lib.fo_lion_fill_chunks(0x1000, 0x1000, 0x1000, 0, None) == 0
+
+
+def test_tune_hook():
+    lib = _lib.load()
+    assert lib.fo_tune_get(b"lion.variant") == -1
+    assert lib.fo_tune_set(b"lion.variant", 3) == 0 and lib.fo_tune_get(b"lion.variant") == 3
+    assert lib.fo_tune_set(b"lion.variant", -1) == 0
+    assert lib.fo_tune_set(b"no.such.key", 1) == -8
+
+
+def test_python_surfaces_validate_like_the_reference():
+    import torch
+
+    from fast_ops.lion.lion_optimizer import Lion
+    from fast_ops.flash_attention.flash_attention import multi_head_attention
+
+    p = [torch.nn.Parameter(torch.zeros(4))]
+    with pytest.raises(RuntimeError, match="expected positive LR"):
+        Lion(p, lr=0.0)
+    with pytest.raises(RuntimeError, match="betas must be between 0 and 1"):
+        Lion(p, betas=(1.5, 0.9))
+    opt = Lion(p, lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
+    assert opt.defaults == {"lr": 1e-4, "betas": (0.9, 0.99), "weight_decay": 0.1}
+    # CPU tensors: there is no CPU path, the call must raise rather than compute something else
+    p[0].grad = torch.ones(4)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        opt.step()
+    q = torch.zeros(1, 1, 8, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        multi_head_attention(q, q, q)
+    with pytest.raises(RuntimeError, match="half-precision"):
+        multi_head_attention(q.float(), q.float(), q.float())

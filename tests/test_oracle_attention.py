@@ -1,0 +1,126 @@
+"""Pins the attention oracle (oracle/attention_oracle.py) on the CPU.
+
+The reference has no golden vectors for this path (tests/test_flash_attention.py asserts nothing,
+tests/test_flash_attention_triton.py:104-142 is differential), so the oracle is pinned against an independent
+library routine (scaled_dot_product_attention, logsumexp), a float64 brute force, closed-form invariants, the
+reference's tile recurrence restated in numpy, and the committed fixture tests/golden/attn_small.npz.
+"""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.attention_oracle import attention_fwd_oracle, online_softmax_tiles
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "attn_small.npz")
+
+
+def _qkv(B, H, M, N, D, seed=0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, M, D, generator=g).to(dtype)
+    k = torch.randn(B, H, N, D, generator=g).to(dtype)
+    v = torch.randn(B, H, N, D, generator=g).to(dtype)
+    return q, k, v
+
+
+def _brute_force(q, k, v, causal, scale):
+    """float64 loops straight from the definition: O_i = sum_j softmax_j(scale q_i.k_j) v_j over allowed j."""
+    q, k, v = (t.double().numpy() for t in (q, k, v))
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    o = np.zeros((B, H, M, D))
+    lse = np.zeros((B, H, M))
+    for b in range(B):
+        for h in range(H):
+            for i in range(M):
+                js = [j for j in range(N) if (not causal) or j <= i]
+                s = np.array([scale * float(np.dot(q[b, h, i], k[b, h, j])) for j in js])
+                mx = s.max()
+                w = np.exp(s - mx)
+                lse[b, h, i] = mx + math.log(w.sum())
+                o[b, h, i] = sum(w[t] * v[b, h, j] for t, j in enumerate(js)) / w.sum()
+    return o, lse
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_against_float64_brute_force(causal):
+    q, k, v = _qkv(1, 2, 13, 13, 8, seed=1)
+    o, lse = attention_fwd_oracle(q, k, v, causal=causal, softmax_scale=0.3)
+    o64, lse64 = _brute_force(q, k, v, causal, 0.3)
+    assert np.allclose(o.numpy(), o64, atol=2e-6, rtol=1e-5)
+    assert np.allclose(lse.numpy(), lse64, atol=2e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(2, 4, 128, 64), (1, 3, 257, 128)])
+def test_against_library_sdpa_and_logsumexp(causal, shape):
+    B, H, S, D = shape
+    q, k, v = _qkv(B, H, S, S, D, seed=2, dtype=torch.bfloat16)
+    o, lse = attention_fwd_oracle(q, k, v, causal=causal, q_chunk=100)
+    scale = 1 / math.sqrt(D)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=causal, scale=scale)
+    assert torch.allclose(o, ref, atol=1e-5, rtol=1e-5)
+    s = (q.float() @ k.float().transpose(-1, -2)) * scale
+    if causal:
+        s = s.masked_fill(torch.ones(S, S, dtype=torch.bool).triu(1), float("-inf"))
+    assert torch.allclose(lse, torch.logsumexp(s, -1), atol=1e-5, rtol=1e-6)
+
+
+def test_invariants():
+    B, H, S, D = 1, 2, 64, 16
+    q, k, v = _qkv(B, H, S, S, D, seed=3)
+    # V == 1 => O == 1
+    o, _ = attention_fwd_oracle(q, k, torch.ones_like(v), causal=True)
+    assert torch.allclose(o, torch.ones_like(o), atol=1e-6)
+    # Q == 0 => O_i = mean of the allowed V rows, LSE_i = ln(#allowed)
+    o, lse = attention_fwd_oracle(torch.zeros_like(q), k, v, causal=True)
+    cm = torch.cumsum(v, dim=2) / torch.arange(1, S + 1).view(1, 1, S, 1)
+    assert torch.allclose(o, cm, atol=1e-5)
+    assert torch.allclose(lse, torch.log(torch.arange(1, S + 1, dtype=torch.float32)).expand(B, H, S), atol=1e-6)
+    o, lse = attention_fwd_oracle(torch.zeros_like(q), k, v, causal=False)
+    assert torch.allclose(o, v.mean(dim=2, keepdim=True).expand_as(o), atol=1e-5)
+    assert torch.allclose(lse, torch.full_like(lse, math.log(S)), atol=1e-6)
+    # causal row 0 sees only key 0
+    o, lse = attention_fwd_oracle(q, k, v, causal=True)
+    assert torch.allclose(o[:, :, 0], v[:, :, 0], atol=1e-6)
+    assert torch.allclose(lse[:, :, 0], (q[:, :, 0] * k[:, :, 0]).sum(-1) / math.sqrt(D), atol=1e-5)
+    # non-causal: permuting the keys (and values with them) changes nothing
+    perm = torch.randperm(S, generator=torch.Generator().manual_seed(9))
+    o1, l1 = attention_fwd_oracle(q, k, v, causal=False)
+    o2, l2 = attention_fwd_oracle(q, k[:, :, perm], v[:, :, perm], causal=False)
+    assert torch.allclose(o1, o2, atol=1e-5) and torch.allclose(l1, l2, atol=1e-5)
+    # exp(scale*qk - LSE) is the softmax: rows sum to 1 and reproduce O
+    s = (q @ k.transpose(-1, -2)) / math.sqrt(D)
+    pr = torch.exp(s - l1.unsqueeze(-1))
+    assert torch.allclose(pr.sum(-1), torch.ones(B, H, S), atol=1e-5)
+    assert torch.allclose(pr @ v, o1, atol=1e-5)
+    # a dominant key selects its value row
+    q2 = torch.zeros(1, 1, 4, D); k2 = torch.zeros(1, 1, 4, D); v2 = torch.randn(1, 1, 4, D)
+    for i in range(4):
+        q2[0, 0, i, i] = 60.0
+        k2[0, 0, (i + 1) % 4, i] = 60.0
+    o, _ = attention_fwd_oracle(q2, k2, v2, causal=False, softmax_scale=1.0)
+    assert torch.allclose(o[0, 0], v2[0, 0, [1, 2, 3, 0]], atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_tile_recurrence_equals_closed_form(causal):
+    """The reference's online recurrence (running reference = lse_i) equals the closed form."""
+    q, k, v = _qkv(1, 1, 384, 384, 32, seed=4)
+    scale = 1 / math.sqrt(32)
+    o, lse = attention_fwd_oracle(q, k, v, causal=causal)
+    o_t, lse_t = online_softmax_tiles(q[0, 0].numpy(), k[0, 0].numpy(), v[0, 0].numpy(), causal, scale)
+    assert np.allclose(o_t, o[0, 0].numpy(), atol=2e-5, rtol=1e-5)
+    assert np.allclose(lse_t, lse[0, 0].numpy(), atol=2e-5, rtol=1e-6)
+
+
+def test_golden_fixture():
+    z = np.load(GOLDEN)
+    to16 = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16)
+    q, k, v = to16(z["q"]), to16(z["k"]), to16(z["v"])
+    for tag, causal in (("full", False), ("causal", True)):
+        o, lse = attention_fwd_oracle(q, k, v, causal=causal, softmax_scale=float(z["scale"]))
+        assert np.allclose(o.numpy(), z[f"o_{tag}"], atol=1e-5, rtol=1e-5)
+        assert np.allclose(lse.numpy(), z[f"lse_{tag}"], atol=1e-5, rtol=1e-6)
