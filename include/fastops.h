@@ -82,7 +82,7 @@ int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
  *     u  = f32(bf16(m * c_b1)) + g * c_1b1
  *     p  = p1 + c_nlr * sign(u)                 sign(+-0) = sign(NaN) = 0
  *     m  = bf16( fma(c_1b2, g, f32(bf16(m * c_b2))) )
- * bf16() is round-to-nearest-even (NaN -> 0x7FC0). The kernel fuses what lion_update_kernel fuses
+ * bf16() is round-to-nearest-even; a NaN stays a quiet NaN whose payload bits are unspecified. The kernel fuses what lion_update_kernel fuses
  * (lion_update.cu:44-106) but keeps the fp32 rounding points of the Python formula instead of half arithmetic.
  */
 typedef struct fo_lion_consts {

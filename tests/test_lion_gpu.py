@@ -52,7 +52,7 @@ def test_single_tensor_bit_exact(n):
     assert torch.equal(gd.cpu(), gr), "gradient must not be written"
 
 
-@pytest.mark.parametrize("variant", list(range(16)))
+@pytest.mark.parametrize("variant", list(range(32)))
 def test_every_kernel_variant_bit_exact(variant):
     n = 5 * 8192 + 77
     p, gr, m = _seeded(n, seed=100 + variant)
@@ -86,7 +86,10 @@ def test_adversarial_values():
     nan = np.isnan(pc)
     assert np.array_equal(np.isnan(got_p), nan)
     assert np.array_equal(got_p.view(np.uint32)[~nan], pc.view(np.uint32)[~nan])
-    assert np.array_equal(got_m, mc)   # NaN momentum is 0x7FC0 on both sides
+    # NaN momentum: only NaN-ness is defined (torch's own scalar and vector conversions write different payloads)
+    m_nan = (mc & 0x7FFF) > 0x7F80
+    assert np.array_equal((got_m & 0x7FFF) > 0x7F80, m_nan)
+    assert np.array_equal(got_m[~m_nan], mc[~m_nan])
 
 
 def test_unaligned_views_take_the_scalar_path():
