@@ -27,6 +27,7 @@ COMMON_FLAGS = [
     "-fPIC",
     "-Wall",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",   # the direct-to-LDS copies name m0, a reserved register, as a clobber
     # packed fp32 instructions stay off for every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]

@@ -27,6 +27,7 @@
 namespace fo {
 
 #define FO_LDS __attribute__((address_space(3)))
+#define FO_GLOBAL __attribute__((address_space(1)))
 
 constexpr int kWaves = 4;
 constexpr int kBM = 32 * kWaves;   // query rows per workgroup
@@ -63,7 +64,24 @@ __device__ __forceinline__ float half_swap(float x) {
   return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
 }
 
-template <typename T, int D, bool CAUSAL>
+// 16 bytes per lane, global -> LDS without passing through registers. LDS receives the 64 lanes' pieces back to back
+// starting at `dst` (wave-uniform); the global address is per lane.
+// (hipcc also parses device functions in its host pass, where GCN assembly cannot be checked: the bodies exist in the
+// device pass only.)
+__device__ __forceinline__ void dma16_uniform_base(const void* base, uint32_t byte_off, FO_LDS void* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"((uint32_t)(uintptr_t)dst), "v"(byte_off), "s"(base) : "memory", "m0");
+#endif
+}
+__device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"((uint32_t)(uintptr_t)dst), "v"(ptr) : "memory", "m0");
+#endif
+}
+
+constexpr float kLazyLog2 = 8.0f;   // how far (in log2 units) a tile maximum may exceed the reference before a rescale
+
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG>
 __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int ROW_BYTES = D * 2;
@@ -79,6 +97,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
   // layout: K0 | K1 | V0 | V1
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // the same, known to the compiler as wave-uniform (DMA operands)
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hh = lane >> 5;
@@ -115,28 +134,50 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     n_tiles = (Sk + kBN - 1) / kBN;
   }
 
-  // ---- direct-to-LDS copy of one K and one V tile: per lane, DMA_PER_WAVE 16-byte pieces of each
-  // piece i of this wave covers tile rows [ (wave*DMA_PER_WAVE + i) * ROWS_PER_DMA, +ROWS_PER_DMA )
-  int dma_row[DMA_PER_WAVE], dma_col[DMA_PER_WAVE];
+  // ---- direct-to-LDS copy of one K and one V tile: per lane, DMA_PER_WAVE 16-byte pieces of each.
+  // Piece i of this wave covers tile rows [(wave*DMA_PER_WAVE + i) * ROWS_PER_DMA, +ROWS_PER_DMA). LDS receives the
+  // 64 lanes' pieces back to back, so the swizzle is applied by choosing which global chunk each lane fetches.
+  // Per-lane byte offsets inside a tile are fixed; a tile's base pointer is wave-uniform.
+  uint32_t k_off[DMA_PER_WAVE], v_off[DMA_PER_WAVE];
 #pragma unroll
   for (int i = 0; i < DMA_PER_WAVE; ++i) {
-    const int row = (wave * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane / CHUNKS;
-    const int phys = lane % CHUNKS;
-    dma_row[i] = row;
-    dma_col[i] = (phys ^ swz<D>(row)) * 8;          // logical chunk -> element offset in the row
+    const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane / CHUNKS;
+    const int col = ((lane % CHUNKS) ^ swz<D>(row)) * 8;     // logical chunk -> element offset in the row
+    k_off[i] = (uint32_t)(row * (int)prm.ks[2] + col) * 2u;
+    v_off[i] = (uint32_t)(row * (int)prm.vs[2] + col) * 2u;
   }
+  // The copies are issued as inline assembly so that the compiler does not track them: with the builtin it makes every
+  // later LDS read it cannot disambiguate wait for ALL outstanding copies (vmcnt(0) in the middle of a tile, i.e.
+  // for the NEXT tile's data). Completion is awaited explicitly, once per tile, before the barrier at the loop top.
+  // The loop contains no other vector-memory instruction, so no compiler-inserted vmcnt wait depends on these.
   auto issue_tile = [&](int tile, int buf) {
     const int key0 = tile * kBN;
     FO_LDS char* kdst = smem + buf * TILE_BYTES;
     FO_LDS char* vdst = smem + (2 + buf) * TILE_BYTES;
+    if (key0 + kBN <= Sk) {
+      const char* ktile = (const char*)(kbase + (int64_t)key0 * prm.ks[2]);
+      const char* vtile = (const char*)(vbase + (int64_t)key0 * prm.vs[2]);
 #pragma unroll
-    for (int i = 0; i < DMA_PER_WAVE; ++i) {
-      const int key = min(key0 + dma_row[i], Sk - 1);        // rows past the end re-read the last key; masked later
-      const T* ksrc = kbase + (int64_t)key * prm.ks[2] + dma_col[i];
-      const T* vsrc = vbase + (int64_t)key * prm.vs[2] + dma_col[i];
-      const int lds_off = (wave * DMA_PER_WAVE + i) * 1024;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ksrc, (FO_LDS void*)(kdst + lds_off), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc, (FO_LDS void*)(vdst + lds_off), 16, 0, 0);
+      for (int i = 0; i < DMA_PER_WAVE; ++i) {
+        const int lds_off = (wave_s * DMA_PER_WAVE + i) * 1024;
+        dma16_uniform_base(ktile, k_off[i], kdst + lds_off);
+        dma16_uniform_base(vtile, v_off[i], vdst + lds_off);
+      }
+    } else {
+      // last, partial tile: rows past the end re-read the last key (masked later). Runs at most once per workgroup;
+      // the opaque copy of the lane id keeps its address arithmetic from being hoisted out of the tile loop, where
+      // it would hold registers for the whole kernel.
+      int lane_here = lane;
+      asm volatile("" : "+v"(lane_here));
+#pragma unroll
+      for (int i = 0; i < DMA_PER_WAVE; ++i) {
+        const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane_here / CHUNKS;
+        const int col = ((lane_here % CHUNKS) ^ swz<D>(row)) * 8;
+        const int key = min(key0 + row, Sk - 1);
+        const int lds_off = (wave_s * DMA_PER_WAVE + i) * 1024;
+        dma16_lane_ptr(kbase + (int64_t)key * prm.ks[2] + col, kdst + lds_off);
+        dma16_lane_ptr(vbase + (int64_t)key * prm.vs[2] + col, vdst + lds_off);
+      }
     }
   };
 
@@ -149,6 +190,10 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const T* qp = qbase + (int64_t)qrow * prm.qs[2] + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *(const vec8*)(qp + 16 * ks);
+    // Consume the fragments here so that the compiler waits for these loads before the loop instead of inside it:
+    // a vmcnt wait inside the loop would also wait for the direct-to-LDS copies in flight, which it does not see.
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[ks]));
   }
 
   f32x16 oacc[DBLK];
@@ -156,7 +201,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
   for (int i = 0; i < DBLK; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.0f;
-  float m_run = -INFINITY;   // running max of the raw (unscaled) scores of this lane's query row
+  float m_run = -INFINITY;   // reference maximum (raw, unscaled scores) of this lane's query row
   float l_run = 0.0f;        // running sum of this lane's half of the keys
   const float c = prm.scale_log2e;
 
@@ -169,9 +214,9 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int buf = tile & 1;
     const int key0 = tile * kBN;
-    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this lane's pieces of tile `tile` have landed in LDS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's pieces of tile `tile` have landed in LDS
     __syncthreads();                        // everyone's pieces have landed; everyone is done reading the other buffer
-    if (tile + 1 < n_tiles) issue_tile(tile + 1, buf ^ 1);
+    if (tile + 1 < n_tiles && (!(DBG & 1) || tile < 1)) issue_tile(tile + 1, buf ^ 1);
 
     // waves whose rows are all above this tile's keys have nothing to do (causal)
     if (CAUSAL && key0 > q0w + 31) continue;
@@ -183,15 +228,22 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     //      MFMAs that consume them, so LDS latency hides behind the previous group's matrix work.
     f32x16 sacc[2];
     {
-      constexpr int GK = KSTEPS < 4 ? KSTEPS : 4;          // k-steps per fragment group
+      // a group = GK fragments = GK/2 k-steps of both key blocks; consecutive MFMAs alternate between the two
+      // accumulators (a dependent MFMA issued back to back costs ~6 extra cycles on this hardware)
+      constexpr int GK = 4;
       constexpr int NG = 2 * KSTEPS / GK;                   // groups per tile
       auto load_group = [&](int g, vec8* dst) {
-        const int kb = (g * GK) / KSTEPS, ks0 = (g * GK) % KSTEPS;
-        const int row = 32 * kb + l32;
-        const int sw = swz<D>(row);
 #pragma unroll
-        for (int i = 0; i < GK; ++i) dst[i] = *(FO_LDS const vec8*)(kt + row * ROW_BYTES + (((2 * (ks0 + i) + hh) ^ sw) * 16));
+        for (int i = 0; i < GK; ++i) {
+          const int kb = i & 1, ks = g * (GK / 2) + (i >> 1);
+          const int row = 32 * kb + l32;
+          dst[i] = *(FO_LDS const vec8*)(kt + row * ROW_BYTES + (((2 * ks + hh) ^ swz<D>(row)) * 16));
+        }
       };
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.0f;
       vec8 fa[GK], fb[GK];
       load_group(0, fa);
 #pragma unroll
@@ -199,59 +251,61 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
         vec8* cur = (g & 1) ? fb : fa;
         vec8* nxt = (g & 1) ? fa : fb;
         if (g + 1 < NG) load_group(g + 1, nxt);
-        const int kb = (g * GK) / KSTEPS, ks0 = (g * GK) % KSTEPS;
 #pragma unroll
-        for (int i = 0; i < GK; ++i) {
-          if (ks0 + i == 0) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.0f;
-          }
-          sacc[kb] = Ops<T>::mfma(cur[i], qf[ks0 + i], sacc[kb]);
-        }
+        for (int i = 0; i < GK; ++i) sacc[i & 1] = Ops<T>::mfma(cur[i], qf[g * (GK / 2) + (i >> 1)], sacc[i & 1]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
 
-    // ---- mask: causal diagonal and keys past the end
+    // ---- mask: causal diagonal and keys past the end. Register r of block kb holds key
+    //      key0 + 32*kb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); it is dead iff key > q or key >= Sk,
+    //      i.e. iff lim + koff(r) > 0 with lim = max(key_base - q, key_base - Sk + 1): one compare against a constant.
     const bool need_mask = (CAUSAL && key0 + kBN - 1 > q0w) || (key0 + kBN > Sk);
     if (need_mask) {
-      const int qi = q0w + l32;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb) {
+        const int key_base = key0 + 32 * kb + 4 * hh;
+        int lim = key_base - Sk + 1;
+        if (CAUSAL) lim = max(lim, key_base - (q0w + l32));
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = key0 + 32 * kb + (r & 3) + 8 * (r >> 2) + 4 * hh;
-          const bool dead = (CAUSAL && key > qi) || key >= Sk;
-          sacc[kb][r] = dead ? -INFINITY : sacc[kb][r];
-        }
+        for (int r = 0; r < 16; ++r) sacc[kb][r] = (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : sacc[kb][r];
+      }
     }
 
-    // ---- online softmax (base-2 domain)
+    // ---- online softmax (base-2 domain) with a lazily updated reference maximum.
+    // exp2 is taken relative to m_run, which is only raised (and O, l rescaled) when some row's tile maximum exceeds it
+    // by more than 2^kLazyLog2; until then P may reach 2^kLazyLog2 instead of 1, which fp32 accumulators and the
+    // half-precision P hold without loss of relative precision. O / l and LSE = m + log(l) do not depend on the
+    // reference, so the result is that of the exact recurrence (flash_attention_triton.py:200-213,241-243) up to rounding.
     float mloc = sacc[0][0];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
     mloc = fmaxf(mloc, half_swap(mloc));
-    const float m_new = fmaxf(m_run, mloc);          // finite from the first tile on: key 0 is never masked
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
-    const float mc = m_new * c;
-    m_run = m_new;
+    const bool raise = LAZY ? (mloc * c > m_run * c + kLazyLog2) : (mloc > m_run);
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+      const float m_new = fmaxf(m_run, mloc);          // finite from the first tile on: key 0 is never masked
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+    }
+    const float mc = m_run * c;
     float psum = 0.0f;
     vec8 pf[4];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -mc));
+        const float p = (DBG & 2) ? sacc[kb][r] : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -mc));
         psum += p;                                     // summed in fp32 before rounding (flash_attention_triton.py:203)
         pf[kb * 2 + (r >> 3)][r & 7] = (T)p;           // rounded to the operand type for P.V (:237)
       }
-    l_run = l_run * alpha + psum;
-#pragma unroll
-    for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+    l_run += psum;
 
     // ---- O^T += V^T P^T : four 16-key steps x DBLK d-blocks, V^T fragments fetched one group ahead
     {
@@ -306,20 +360,33 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
   }
 }
 
-template <typename T, int D>
-static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG>
+static int launch_one(const AttnParams& p, hipStream_t stream) {
   const size_t lds = 4 * (size_t)kBN * D * 2;
   const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
-  if (causal) {
-    static bool once = (hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
-    (void)once;
-    attn_fwd_kernel<T, D, true><<<grid, kWaves * 64, lds, stream>>>(p);
-  } else {
-    static bool once = (hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
-    (void)once;
-    attn_fwd_kernel<T, D, false><<<grid, kWaves * 64, lds, stream>>>(p);
-  }
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (attr != hipSuccess) return FO_ERR_LAUNCH;
+  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG><<<grid, kWaves * 64, lds, stream>>>(p);
   return launch_status();
+}
+
+// variant bit 0: 1 = exact (eager) rescale instead of the lazy one. Variants 2..7 are timing ablations that produce
+// WRONG results (bit 1: keep re-using the first tiles instead of copying new ones; bit 2: no exponentials).
+template <typename T, int D>
+static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
+  const int v = g_attn_variant < 0 ? 0 : g_attn_variant;
+  if (D == 128 && causal && sizeof(T) == 2) {
+    switch (v >> 1) {
+      case 1: return launch_one<T, D, true, true, 1>(p, stream);
+      case 2: return launch_one<T, D, true, true, 2>(p, stream);
+      case 3: return launch_one<T, D, true, true, 3>(p, stream);
+      default: break;
+    }
+  }
+  const bool lazy = (v & 1) == 0;
+  if (causal) return lazy ? launch_one<T, D, true, true, 0>(p, stream) : launch_one<T, D, true, false, 0>(p, stream);
+  return lazy ? launch_one<T, D, false, true, 0>(p, stream) : launch_one<T, D, false, false, 0>(p, stream);
 }
 
 }  // namespace fo
@@ -348,7 +415,7 @@ extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o,
   if (os[1] == 0 && H > 1) return FO_ERR_BAD_STRIDE;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15u) return FO_ERR_MISALIGNED;
   if (lse && ((uintptr_t)lse & 3u)) return FO_ERR_MISALIGNED;
-  if (!(softmax_scale == softmax_scale)) return FO_ERR_BAD_SHAPE;
+  if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;   // also rejects NaN
 
   AttnParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;

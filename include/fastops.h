@@ -67,7 +67,8 @@ int fo_tune_get(const char* key);
  *   causal       non-zero: query i attends keys j <= i (top-left aligned, attention_ref.py:54-58)
  *   dtype        FO_DTYPE_F16 or FO_DTYPE_BF16, for q, k, v and o alike
  *
- * Requirements checked here: D in {64, 128}; Sq, Sk >= 1; base pointers and row strides multiples of 16 bytes.
+ * Requirements checked here: D in {64, 128}; Sq, Sk >= 1; softmax_scale finite and > 0; base pointers and row strides
+ * multiples of 16 bytes.
  */
 int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                 int B, int H, int Sq, int Sk, int D,

@@ -66,6 +66,7 @@ def test_attn_argument_validation_without_device():
     assert call(ks=bad) == -5
     assert call(q=0x1008) == -6
     assert call(scale=float("nan")) == -4
+    assert call(scale=0.0) == -4 and call(scale=-1.0) == -4
 
 
 def test_lion_argument_validation_without_device():
