@@ -22,6 +22,8 @@
 //     (32 rows x one chunk) and the V reads (4 rows x 4 chunks) are free of bank conflicts.
 //   * Workgroup order: heads are dealt to the 8 XCDs (workgroup ids round-robin over XCDs), each XCD walks one head
 //     at a time with its heaviest (last) causal query blocks first, so an XCD's L2 holds the K/V it is streaming.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace fo {
@@ -215,7 +217,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const int buf = tile & 1;
     const int key0 = tile * kBN;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's pieces of tile `tile` have landed in LDS
-    __syncthreads();                        // everyone's pieces have landed; everyone is done reading the other buffer
+    if (!(DBG & 4)) __syncthreads();        // everyone's pieces have landed; everyone is done reading the other buffer
     if (tile + 1 < n_tiles && (!(DBG & 1) || tile < 1)) issue_tile(tile + 1, buf ^ 1);
 
     // waves whose rows are all above this tile's keys have nothing to do (causal)
@@ -360,6 +362,399 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
   }
 }
 
+// =====================================================================================================================
+// Pipelined kernel: 8 waves x 32 query rows = 256 rows per workgroup, one workgroup per CU (two waves per SIMD, at
+// most 256 VGPRs each, no AccVGPRs), K and V in four-slot LDS rings (128 KiB at D = 128) filled two tiles ahead.
+// Inside a wave the work is cut into 32-key sub-tiles and software-pipelined so that the MFMA pipe and the VALU
+// overlap within ONE wave instead of relying on the other wave's phase:
+//     phase A(s):  S(s+1) = K Q^T  (8 MFMAs)   interleaved with   P(s) = exp2(S(s) c - m c), row sums   (VALU)
+//     phase B(s):  O += V^T P(s)^T (8 MFMAs)   interleaved with   mask + row max of S(s+1)              (VALU)
+// followed by the (rare) raise of the reference maximum. LDS fragments are fetched one batch (4 MFMAs) ahead through
+// two register buffers, across phase and tile boundaries.
+constexpr int kPipeBM = 256;
+constexpr int kRing = 4;
+constexpr int SG_VALU = 0x2, SG_MFMA = 0x8, SG_DS_READ = 0x100, SG_TRANS = 0x400;   // sched_group_barrier masks
+
+// scheduling recipe for one batch: the LDS reads of the next batch first, then 4*NG x (1 MFMA, NV VALU, NT transcendental)
+template <bool ON, int NG, int NDS, int NV, int NT>
+__device__ __forceinline__ void sched_batch() {
+  if constexpr (ON) {
+    if constexpr (NDS > 0) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, NDS, 0);
+#pragma unroll
+    for (int q = 0; q < 4 * NG; ++q) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      if constexpr (NV > 0) __builtin_amdgcn_sched_group_barrier(SG_VALU, NV, 0);
+      if constexpr (NT > 0) __builtin_amdgcn_sched_group_barrier(SG_TRANS, NT, 0);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+template <typename T, int D, bool CAUSAL, int SCHED, int NG>
+__global__ void __launch_bounds__(kPipeBM / (32 * NG) * 64) attn_fwd_pipe_kernel(const AttnParams prm) {
+  constexpr int NWAVES = kPipeBM / (32 * NG);     // 8 waves x 32 rows, or 4 waves x 64 rows (two row groups per wave)
+  typedef typename Ops<T>::vec8 vec8;
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CHUNKS = ROW_BYTES / 16;
+  constexpr int TILE_BYTES = kBN * ROW_BYTES;
+  constexpr int KSTEPS = D / 16;                 // MFMAs of one sub-tile's Q K^T
+  constexpr int DBLK = D / 32;
+  constexpr int NB = KSTEPS / 4;                 // batches (of 4 MFMAs) per phase: 2 at D = 128, 1 at D = 64
+  constexpr int DMA_PER_WAVE = TILE_BYTES / 1024 / NWAVES;
+  constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;
+  static_assert(2 * DBLK == KSTEPS && DMA_PER_WAVE >= 1, "tile shape");
+
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;    // K ring (kRing tiles) | V ring (kRing tiles)
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int lane = tid & 63;
+  const int l32 = lane & 31;
+  const int hh = lane >> 5;
+  const int L16 = lane & 15;
+  const int g16 = (lane >> 4) & 1;
+
+  const int n_bh = prm.B * prm.H;
+  int bh, qblk;
+  {
+    const int id = blockIdx.x;
+    if ((n_bh & 7) == 0) {
+      const int x = id & 7, j = id >> 3;
+      bh = x + 8 * (j / prm.n_qblk);
+      qblk = prm.n_qblk - 1 - (j % prm.n_qblk);
+    } else {
+      bh = id % n_bh;
+      qblk = prm.n_qblk - 1 - id / n_bh;
+    }
+  }
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int q0 = qblk * kPipeBM;
+  const int q0w = q0 + wave_s * 32 * NG;
+  const int Sq = prm.Sq, Sk = prm.Sk;
+  const T* __restrict__ qbase = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  const T* __restrict__ kbase = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1];
+  const T* __restrict__ vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
+
+  int n_tiles, n_w;                       // tiles the workgroup walks / tiles in which this wave has unmasked keys
+  if constexpr (CAUSAL) {
+    n_tiles = (min(Sk, q0 + kPipeBM) + kBN - 1) / kBN;
+    n_w = min(n_tiles, (q0w + 32 * NG - 1) / kBN + 1);
+  } else {
+    n_tiles = (Sk + kBN - 1) / kBN;
+    n_w = n_tiles;
+  }
+
+  // ---- global -> LDS copies
+  uint32_t k_off[DMA_PER_WAVE], v_off[DMA_PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < DMA_PER_WAVE; ++i) {
+    const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane / CHUNKS;
+    const int col = ((lane % CHUNKS) ^ swz<D>(row)) * 8;
+    k_off[i] = (uint32_t)(row * (int)prm.ks[2] + col) * 2u;
+    v_off[i] = (uint32_t)(row * (int)prm.vs[2] + col) * 2u;
+  }
+  // one tile of K (ring 0) or V (ring 1) into slot tile % kRing
+  auto issue = [&](const T* base, int64_t stride, const uint32_t* off, int tile, int ring) {
+    const int key0 = tile * kBN;
+    FO_LDS char* dst = smem + (kRing * ring + (tile & (kRing - 1))) * TILE_BYTES;
+    if (key0 + kBN <= Sk) {
+      const char* src = (const char*)(base + (int64_t)key0 * stride);
+#pragma unroll
+      for (int i = 0; i < DMA_PER_WAVE; ++i) dma16_uniform_base(src, off[i], dst + (wave_s * DMA_PER_WAVE + i) * 1024);
+    } else {
+      int lane_here = lane;                            // (opaque: keeps this rare path's address math inside it)
+      asm volatile("" : "+v"(lane_here));
+#pragma unroll
+      for (int i = 0; i < DMA_PER_WAVE; ++i) {
+        const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane_here / CHUNKS;
+        const int col = ((lane_here % CHUNKS) ^ swz<D>(row)) * 8;
+        const int key = min(key0 + row, Sk - 1);       // rows past the end re-read the last key (masked later)
+        dma16_lane_ptr(base + (int64_t)key * stride + col, dst + (wave_s * DMA_PER_WAVE + i) * 1024);
+      }
+    }
+  };
+  // batch(t), issued at the top of tile t: K(t+3) and V(t+2). Returns the number of copies this lane issued.
+  auto issue_batch = [&](int t) -> int {
+    int n = 0;
+    if (t + 3 < n_tiles && t + 3 >= 0) { issue(kbase, prm.ks[2], k_off, t + 3, 0); n += DMA_PER_WAVE; }
+    if (t + 2 < n_tiles && t + 2 >= 0) { issue(vbase, prm.vs[2], v_off, t + 2, 1); n += DMA_PER_WAVE; }
+    return n;
+  };
+  issue_batch(-3);
+  issue_batch(-2);
+  int last_batch = issue_batch(-1);
+
+  // ---- Q^T fragments (B operand of S^T = K Q^T)
+  vec8 qf[NG][KSTEPS];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const int qrow = min(q0w + 32 * g + l32, Sq - 1);
+    const T* qp = qbase + (int64_t)qrow * prm.qs[2] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[g][ks] = *(const vec8*)(qp + 16 * ks);
+  }
+#pragma unroll
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[g][ks]));   // wait for Q here, never inside the loop
+
+  f32x16 oacc[NG][DBLK];
+#pragma unroll
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[g][i][r] = 0.0f;
+  f32x16 Sacc[NG];             // scores of the sub-tile being produced (MFMA accumulators)
+  f32x16 sv[NG];               // scores of the sub-tile being consumed: copied out of Sacc, masked
+  vec8 pf[NG][2];              // P of the sub-tile being multiplied with V (two 16-key steps)
+  vec8 FB[2][4];               // LDS fragment batches: current and next (each fragment feeds NG MFMAs)
+  float m_run[NG], l_run[NG], mloc[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) { m_run[g] = -INFINITY; l_run[g] = 0.0f; mloc[g] = -INFINITY; }
+  const float c = prm.scale_log2e;
+
+  // Held in registers for the whole kernel: 8 byte offsets for K (one per k-step) and 2 x DBLK for V^T; everything else
+  // about a fragment address (ring slot, sub-tile half, 16-key step) is a wave-uniform or compile-time addend.
+  uint32_t koffs[KSTEPS], voffs0[DBLK], voffs1[DBLK];
+  {
+    const int ksw = swz<D>(l32);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) koffs[ks] = (uint32_t)(l32 * ROW_BYTES + (((2 * ks + hh) ^ ksw) * 16));
+    const int vrow0 = 4 * hh + (L16 >> 2);
+    const int vsw0 = swz<D>(vrow0), vsw1 = swz<D>(vrow0 + 8);
+    const int vsub = (L16 & 1) * 8;
+    const int vchunk = 2 * g16 + ((L16 & 3) >> 1);
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db) {
+      voffs0[db] = (uint32_t)(vrow0 * ROW_BYTES + vsub + (((4 * db + vchunk) ^ vsw0) * 16));
+      voffs1[db] = (uint32_t)((vrow0 + 8) * ROW_BYTES + vsub + (((4 * db + vchunk) ^ vsw1) * 16));
+    }
+  }
+  auto read_k4 = [&](vec8 (&dst)[4], FO_LDS const char* kt, int hf, int ks0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = *(FO_LDS const vec8*)(kt + hf * 32 * ROW_BYTES + koffs[ks0 + i]);
+  };
+  // four V^T fragments: batch bi of sub-tile half hf. At D = 128: t = 2*hf + bi, db = 0..3. At D = 64: t = 2*hf + i/2, db = i%2.
+  auto read_v4 = [&](vec8 (&dst)[4], FO_LDS const char* vt, int hf, int bi) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = (DBLK == 4) ? 2 * hf + bi : 2 * hf + (i >> 1);
+      const int db = (DBLK == 4) ? i : (i & 1);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(vt + 16 * t * ROW_BYTES + voffs0[db]));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(vt + 16 * t * ROW_BYTES + voffs1[db]));
+      dst[i] = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  };
+  auto k_slot = [&](int tile) -> FO_LDS const char* { return smem + (tile & (kRing - 1)) * TILE_BYTES; };
+  auto v_slot = [&](int tile) -> FO_LDS const char* { return smem + (kRing + (tile & (kRing - 1))) * TILE_BYTES; };
+
+  // ---- VALU pieces
+  // exponentials of elements [e0, e1) of sv -> pf, psum
+  auto exp_part = [&](const float (&mc)[NG], float (&psum)[NG], int e0, int e1) {
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int e = e0; e < e1; ++e) {
+        const float x = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[g][e], c, -mc[g]));
+        psum[g] += x;                              // summed in fp32 before rounding (flash_attention_triton.py:203)
+        pf[g][e >> 3][e & 7] = (T)x;               // rounded to the operand type for P.V (:237)
+      }
+  };
+  // elements [e0, e1) of the sub-tile just produced (half hf of tile): copy out of the accumulators, mask, fold into the
+  // row max. The mask is applied unconditionally (two VALU operations per element, hidden behind phase B's MFMAs): a
+  // branch on "this tile needs a mask" would split the straight-line block that the MFMA/VALU interleave relies on.
+  // Register r holds key key_base + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); it is dead iff key > q or key >= Sk,
+  // i.e. iff lim + koff(r) > 0 with lim = max(key_base - q, key_base - Sk + 1).
+  auto max_part = [&](int tile, int hf, int e0, int e1) {
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const int key_base = tile * kBN + 32 * hf + 4 * hh;
+      int lim = key_base - Sk + 1;
+      if (CAUSAL) lim = max(lim, key_base - (q0w + 32 * g + l32));
+#pragma unroll
+      for (int r = e0; r < e1; ++r) sv[g][r] = (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : Sacc[g][r];
+#pragma unroll
+      for (int r = e0; r < e1; r += 2) mloc[g] = fmaxf(fmaxf(mloc[g], sv[g][r]), sv[g][r + 1]);
+    }
+  };
+  // finish the row max, raise the reference maximum where needed (lazily), rescale O and l
+  auto settle = [&]() {
+    bool raise = false;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      mloc[g] = fmaxf(mloc[g], half_swap(mloc[g]));
+      raise = raise || (mloc[g] * c > m_run[g] * c + kLazyLog2);
+    }
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const float m_new = fmaxf(m_run[g], mloc[g]);    // finite from the first sub-tile on: key 0 is never masked
+        const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * c);
+        m_run[g] = m_new;
+        l_run[g] *= alpha;
+#pragma unroll
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[g][i][r] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < NG; ++g) mloc[g] = -INFINITY;
+  };
+
+  // ---- one full step. On entry FB[0] holds the first K batch of sub-tile (tq, hq).
+  //   phase A: Sacc = K(tq, hq) Q^T       ||  P = exp2(sv c - m c)                 (sv = sub-tile (te, he), the previous one)
+  //   phase B: O += V(te, he)^T P^T       ||  sv = mask(Sacc), row max
+  //   then settle; on exit FB[0] holds the first K batch of the sub-tile after (tq, hq) (garbage past the end: unused).
+  auto full_step = [&](int tq, int hq, int te, int he) {
+    FO_LDS const char* kt = k_slot(tq);
+    FO_LDS const char* vt = v_slot(te);
+    FO_LDS const char* kt_next = hq ? k_slot(tq + 1) : kt;
+    float mc[NG], psum[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      mc[g] = m_run[g] * c;
+      psum[g] = 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) Sacc[g][r] = 0.0f;
+    }
+    // phase A
+#pragma unroll
+    for (int bi = 0; bi < NB; ++bi) {
+      if (bi + 1 < NB) read_k4(FB[(bi + 1) & 1], kt, hq, 4 * (bi + 1));
+      else read_v4(FB[(bi + 1) & 1], vt, he, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < NG; ++g) Sacc[g] = Ops<T>::mfma(FB[bi & 1][i], qf[g][4 * bi + i], Sacc[g]);
+      exp_part(mc, psum, bi * (16 / NB), (bi + 1) * (16 / NB));
+      if (bi + 1 < NB) sched_batch<SCHED != 0, NG, 4, (16 / NB) * 5 / 8 + 1, (16 / NB) / 4>();
+      else sched_batch<SCHED != 0, NG, 8, (16 / NB) * 5 / 8 + 1, (16 / NB) / 4>();
+    }
+#pragma unroll
+    for (int g = 0; g < NG; ++g) l_run[g] += psum[g];
+    // phase B (fragment buffers continue to alternate: batch NB of this step sits in FB[NB & 1])
+#pragma unroll
+    for (int bi = 0; bi < NB; ++bi) {
+      const int cur = (NB + bi) & 1;
+      if (bi + 1 < NB) read_v4(FB[cur ^ 1], vt, he, bi + 1);
+      else read_k4(FB[cur ^ 1], kt_next, hq ^ 1, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = (DBLK == 4) ? bi : (i >> 1);       // 16-key step inside the sub-tile
+        const int db = (DBLK == 4) ? i : (i & 1);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) oacc[g][db] = Ops<T>::mfma(FB[cur][i], pf[g][t], oacc[g][db]);
+      }
+      max_part(tq, hq, bi * (16 / NB), (bi + 1) * (16 / NB));
+      if (bi + 1 < NB) sched_batch<SCHED != 0, NG, 8, (16 / NB) * 5 / 8 + 1, 0>();
+      else sched_batch<SCHED != 0, NG, 4, (16 / NB) * 5 / 8 + 1, 0>();
+    }
+    settle();
+  };
+  static_assert(NB == 2 || NB == 1, "fragment buffer parity below assumes one or two batches per phase");
+
+  // ---- first sub-tile alone: Sacc = K(0, 0) Q^T, copy out, mask, max, settle; leaves the next K batch in FB[0]
+  auto first_step = [&]() {
+    FO_LDS const char* kt = k_slot(0);
+    read_k4(FB[0], kt, 0, 0);
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) Sacc[g][r] = 0.0f;
+#pragma unroll
+    for (int bi = 0; bi < NB; ++bi) {
+      if (bi + 1 < NB) read_k4(FB[(bi + 1) & 1], kt, 0, 4 * (bi + 1));
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < NG; ++g) Sacc[g] = Ops<T>::mfma(FB[bi & 1][i], qf[g][4 * bi + i], Sacc[g]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    read_k4(FB[0], kt, 1, 0);
+    max_part(0, 0, 0, 16);
+    settle();
+  };
+  // ---- last sub-tile (te, he) of this wave alone: P = exp2(sv ...), O += V^T P^T
+  auto last_step = [&](int te, int he) {
+    FO_LDS const char* vt = v_slot(te);
+    float mc[NG], psum[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) { mc[g] = m_run[g] * c; psum[g] = 0.0f; }
+    read_v4(FB[0], vt, he, 0);
+    exp_part(mc, psum, 0, 16);
+#pragma unroll
+    for (int g = 0; g < NG; ++g) l_run[g] += psum[g];
+#pragma unroll
+    for (int bi = 0; bi < NB; ++bi) {
+      if (bi + 1 < NB) read_v4(FB[(bi + 1) & 1], vt, he, bi + 1);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = (DBLK == 4) ? bi : (i >> 1);
+        const int db = (DBLK == 4) ? i : (i & 1);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) oacc[g][db] = Ops<T>::mfma(FB[bi & 1][i], pf[g][t], oacc[g][db]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // ---- tile loop. Iteration j: [S(j,0) || P(j-1,1)] [PV(j-1,1) || max(j,0)] [S(j,1) || P(j,0)] [PV(j,0) || max(j,1)]
+  // reads K(j), V(j-1), V(j). Batches up to (j-2) must have landed: K(j+1) and V(j) among them.
+  for (int j = 0; j < n_tiles; ++j) {
+    if (last_batch >= 2 * DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
+    else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    last_batch = issue_batch(j);
+    if (j < n_w) {
+      if (j == 0) first_step();
+      else full_step(j, 0, j - 1, 1);
+      full_step(j, 1, j, 0);
+    } else if (j == n_w) {
+      last_step(j - 1, 1);
+    }
+  }
+  if (n_w == n_tiles) last_step(n_tiles - 1, 1);
+
+  // ---- epilogue: normalise, write O and LSE
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const float l_tot = l_run[g] + half_swap(l_run[g]);
+    const float inv = 1.0f / l_tot;
+    const int qi = q0w + 32 * g + l32;
+    if (qi < Sq) {
+      T* op = (T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)qi * prm.os[2];
+#pragma unroll
+      for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          typedef __attribute__((ext_vector_type(4))) T vec4;
+          vec4 o4;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) o4[u] = (T)(oacc[g][db][rg * 4 + u] * inv);
+          *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
+        }
+      if (prm.lse != nullptr && hh == 0)
+        prm.lse[(int64_t)bh * Sq + qi] = (m_run[g] * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+    }
+  }
+}
+
+template <typename T, int D, bool CAUSAL, int SCHED, int NG>
+static int launch_pipe(AttnParams p, hipStream_t stream) {
+  const size_t lds = 2 * (size_t)kRing * kBN * D * 2;
+  p.n_qblk = (p.Sq + kPipeBM - 1) / kPipeBM;
+  const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_pipe_kernel<T, D, CAUSAL, SCHED, NG>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (attr != hipSuccess) return FO_ERR_LAUNCH;
+  attn_fwd_pipe_kernel<T, D, CAUSAL, SCHED, NG><<<grid, kPipeBM / (32 * NG) * 64, lds, stream>>>(p);
+  return launch_status();
+}
+
 template <typename T, int D, bool CAUSAL, bool LAZY, int DBG>
 static int launch_one(const AttnParams& p, hipStream_t stream) {
   const size_t lds = 4 * (size_t)kBN * D * 2;
@@ -376,11 +771,17 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
   const int v = g_attn_variant < 0 ? 0 : g_attn_variant;
+  if (v == 16) return causal ? launch_pipe<T, D, true, 0, 1>(p, stream) : launch_pipe<T, D, false, 0, 1>(p, stream);
+  if (v == 17) return causal ? launch_pipe<T, D, true, 1, 1>(p, stream) : launch_pipe<T, D, false, 1, 1>(p, stream);
+  if (v == 18) return causal ? launch_pipe<T, D, true, 0, 2>(p, stream) : launch_pipe<T, D, false, 0, 2>(p, stream);
+  if (v == 19) return causal ? launch_pipe<T, D, true, 1, 2>(p, stream) : launch_pipe<T, D, false, 1, 2>(p, stream);
   if (D == 128 && causal && sizeof(T) == 2) {
     switch (v >> 1) {
       case 1: return launch_one<T, D, true, true, 1>(p, stream);
       case 2: return launch_one<T, D, true, true, 2>(p, stream);
       case 3: return launch_one<T, D, true, true, 3>(p, stream);
+      case 4: return launch_one<T, D, true, true, 5>(p, stream);
+      case 5: return launch_one<T, D, true, true, 7>(p, stream);
       default: break;
     }
   }
