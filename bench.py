@@ -21,6 +21,16 @@ PEAK_MFMA_TFLOPS = 2500.0     # MI355X dense bf16/fp16
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
 
+def _measured_traffic(key):
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload (the runs and the
+    scaling against a plain copy are in profiles/hbm_traffic_pmc_*.txt); None when that file is absent."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            return json.load(f).get(key)
+    except OSError:
+        return None
+
+
 def _events(n):
     import torch
 
@@ -69,24 +79,30 @@ def bench_attention(steps, warmup, cpu_baseline):
         "ms_per_step": ms_step,
         "roofline": {
             "bound": "mfma", "achieved": flops / (ms_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-            "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": None,
+            "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": _measured_traffic("attn"),
             "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "flops_per_launch": flops,
         },
         "workload": f"attention fwd B={B} H={H} S={S} D={D} bf16 causal, scale 1/sqrt({D})",
     }
     if cpu_baseline:
-        # bounded sample: ONE (batch, head) slice of the same shape through the oracle's fp32 vanilla path on all host cores
+        # bounded sample: all (batch, head) slices of the same workload through the oracle's fp32 vanilla path on all host
+        # cores, stopped after about 15 s; the rate is that of the slices that were finished
         from oracle.attention_oracle import attention_fwd_oracle
 
         torch.set_num_threads(os.cpu_count())
-        qs, ks, vs = (t[:1, :1].cpu() for t in (q, k, v))
-        attention_fwd_oracle(qs[:, :, :1024], ks[:, :, :1024], vs[:, :, :1024], causal=True, softmax_scale=scale)   # warm-up
-        t0 = time.perf_counter()
-        attention_fwd_oracle(qs, ks, vs, causal=True, softmax_scale=scale)
+        qc, kc, vc = (t.cpu() for t in (q, k, v))
+        attention_fwd_oracle(qc[:1, :1, :1024], kc[:1, :1, :1024], vc[:1, :1, :1024], causal=True, softmax_scale=scale)   # warm-up
+        n_sl, t0 = 0, time.perf_counter()
+        for bb in range(B):
+            for hh in range(H):
+                if time.perf_counter() - t0 > 15.0:
+                    break
+                attention_fwd_oracle(qc[bb:bb + 1, hh:hh + 1], kc[bb:bb + 1, hh:hh + 1], vc[bb:bb + 1, hh:hh + 1], causal=True, softmax_scale=scale)
+                n_sl += 1
         dt = time.perf_counter() - t0
         res["cpu_baseline"] = {
-            "value": 2.0 * S * S * D / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 of {B * H} (batch, head) slices of the same shape, fp32 vanilla softmax(QK^T)V on the host, {dt:.2f} s",
+            "value": n_sl * 2.0 * S * S * D / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{n_sl} of {B * H} (batch, head) slices of the same shape, fp32 vanilla softmax(QK^T)V on the host, {dt:.2f} s",
         }
     return res
 
@@ -112,28 +128,31 @@ def bench_lion(steps, warmup, cpu_baseline):
         "value": nbytes / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms_step, "dtype": "f32 params/grads, bf16 momentum",
         "roofline": {
             "bound": "hbm", "achieved": nbytes / (ms_kernel * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": nbytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+            "frac": nbytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": _measured_traffic("lion"),
             "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "bytes_per_launch": nbytes,
         },
         "workload": f"fused Lion step, {len(shapes)} tensors (39 x 2048x8192 + 39 x 8192x2048) = {n_params} fp32 params, bf16 momentum",
     }
     if cpu_baseline:
-        # bounded sample: one 2048x8192 tensor (1/78 of the workload) through the four reference statements on all host cores
+        # bounded sample: 8 of the 78 tensors (134,217,728 parameters) through the four reference statements on all host
+        # cores, 3 steps
         from oracle.lion_oracle import lion_step_torch
 
         torch.set_num_threads(os.cpu_count())
-        p = params[0].detach().cpu().clone()
-        g = params[0].grad.cpu().clone()
-        m = opt.state[params[0]]["exp_avg"].cpu().clone()
-        lion_step_torch([p], [g], [m], hp["lr"], hp["betas"], hp["weight_decay"])     # warm-up
+        n_t = 8
+        ps = [params[i].detach().cpu().clone() for i in range(n_t)]
+        gs = [params[i].grad.cpu().clone() for i in range(n_t)]
+        ms = [opt.state[params[i]]["exp_avg"].cpu().clone() for i in range(n_t)]
+        lion_step_torch(ps, gs, ms, hp["lr"], hp["betas"], hp["weight_decay"])     # warm-up
         reps = 3
         t0 = time.perf_counter()
         for _ in range(reps):
-            lion_step_torch([p], [g], [m], hp["lr"], hp["betas"], hp["weight_decay"])
+            lion_step_torch(ps, gs, ms, hp["lr"], hp["betas"], hp["weight_decay"])
         dt = (time.perf_counter() - t0) / reps
+        n_el = sum(p.numel() for p in ps)
         res["cpu_baseline"] = {
-            "value": 16.0 * p.numel() / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"1 of 78 tensors (2048x8192), vanilla 4-statement PyTorch Lion step on the host, {dt * 1e3:.1f} ms per step",
+            "value": 16.0 * n_el / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{n_t} of 78 tensors ({n_el} parameters), vanilla 4-statement PyTorch Lion step on the host, {dt * 1e3:.1f} ms per step, {reps} steps",
         }
     del opt, params
     torch.cuda.empty_cache()
@@ -145,7 +164,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--path", choices=["both", "attn", "lion"], default="both")
+    ap.add_argument("--path", choices=["both", "attn", "lion", "copy"], default="both",
+                    help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -159,6 +179,15 @@ def main():
     from fast_ops_amd import _lib
 
     _lib.load()   # fail loudly when the HIP library is missing
+    if args.path == "copy":
+        n = 1 << 30
+        src = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": 4 * n, "copy_bytes_written": 4 * n, "launches": args.warmup + args.steps}))
+        return
     cpu = not args.no_cpu_baseline
     attn = bench_attention(args.steps, args.warmup, cpu) if args.path in ("both", "attn") else None
     lion = bench_lion(args.steps, args.warmup, cpu) if args.path in ("both", "lion") else None
