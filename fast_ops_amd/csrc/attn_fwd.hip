@@ -363,57 +363,121 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
 }
 
 // =====================================================================================================================
-// Pipelined kernel: 8 waves x 32 query rows = 256 rows per workgroup, one workgroup per CU (two waves per SIMD, at
-// most 256 VGPRs each, no AccVGPRs), K and V in four-slot LDS rings (128 KiB at D = 128) filled two tiles ahead.
-// Inside a wave the work is cut into 32-key sub-tiles and software-pipelined so that the MFMA pipe and the VALU
-// overlap within ONE wave instead of relying on the other wave's phase:
-//     phase A(s):  S(s+1) = K Q^T  (8 MFMAs)   interleaved with   P(s) = exp2(S(s) c - m c), row sums   (VALU)
-//     phase B(s):  O += V^T P(s)^T (8 MFMAs)   interleaved with   mask + row max of S(s+1)              (VALU)
-// followed by the (rare) raise of the reference maximum. LDS fragments are fetched one batch (4 MFMAs) ahead through
-// two register buffers, across phase and tile boundaries.
-constexpr int kPipeBM = 256;
+// Wide kernel: 4 waves x 64 query rows = 256 rows per workgroup, one workgroup per CU, ONE wave per SIMD with the
+// whole register file (256 VGPRs for operands, scores and softmax state + the 128 accumulator registers of O^T in
+// AGPRs). K and V tiles in four-slot LDS rings (128 KiB at D = 128) filled two tiles ahead.
+//
+// Measured on MI355X: a SIMD overlaps MFMA and VALU work only when the two alternate INSIDE a wave (about six plain
+// VALU operations, or three transcendentals, issue for free behind each 32x32x16 MFMA); MFMA and VALU work of two
+// different waves on one SIMD mostly serialise. So one wave per SIMD does everything, 64 rows wide (every K / V^T
+// fragment read from LDS feeds two MFMAs, halving LDS traffic per flop), software-pipelined three deep over 32-key
+// sub-tiles, with the instruction stream laid out as micro-groups of ONE MFMA plus its share of LDS reads and
+// softmax arithmetic, fenced so that the compiler keeps that order:
+//     step(s):   S(s+1) = K Q^T          16 MFMAs  \  alternating, 32 micro-groups at D = 128
+//                O += V^T P(s-1)^T       16 MFMAs  /
+//                row max of S(s), new reference maximum, P(s) = exp2(S(s) c - m c), row sums   (VALU, spread over all)
+// The (rare) rescale of O by 2^(old reference - new reference) is applied at the end of the step, after P(s-1) V has
+// been accumulated with the old reference and before P(s) V is.
+//
+// The MFMAs are issued as inline assembly with explicit register classes: accumulators of O^T updated in place in
+// AGPRs, scores in VGPRs. (Left to choose, the compiler puts both in AGPRs, updates them out of place and copies.)
+// Two hazards the compiler can no longer see are kept by construction. A VALU read of an MFMA result needs 11 wait
+// states after an 8-pass MFMA: at least two further MFMAs (8 wait states each) or explicit s_nop separate the last
+// write of a score or accumulator register from its first VALU read. An MFMA source register written by a VALU
+// instruction (measured: also by v_accvgpr_read, which the compiler uses for values it parks in AGPRs) needs two wait
+// states before the MFMA reads it: every MFMA carries them in front.
+constexpr int kWideBM = 256;       // query rows per workgroup: 8 waves x 32 rows (QB = 1) or 4 waves x 64 rows (QB = 2)
 constexpr int kRing = 4;
-constexpr int SG_VALU = 0x2, SG_MFMA = 0x8, SG_DS_READ = 0x100, SG_TRANS = 0x400;   // sched_group_barrier masks
+constexpr float kLargeRowSum = 4096.0f;   // a lane's 16-key row sum above this means some P exceeded 2^8: time to move the reference
 
-// scheduling recipe for one batch: the LDS reads of the next batch first, then 4*NG x (1 MFMA, NV VALU, NT transcendental)
-template <bool ON, int NG, int NDS, int NV, int NT>
-__device__ __forceinline__ void sched_batch() {
-  if constexpr (ON) {
-    if constexpr (NDS > 0) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, NDS, 0);
-#pragma unroll
-    for (int q = 0; q < 4 * NG; ++q) {
-      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-      if constexpr (NV > 0) __builtin_amdgcn_sched_group_barrier(SG_VALU, NV, 0);
-      if constexpr (NT > 0) __builtin_amdgcn_sched_group_barrier(SG_TRANS, NT, 0);
-    }
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+template <typename T> struct AsmMfma;
+#if defined(__HIP_DEVICE_COMPILE__)
+#define FO_MFMA_BODY(MNEMONIC)                                                                                          \
+  /* acc (VGPRs) = a b */                                                                                               \
+  static __device__ __forceinline__ void v_init(f32x16& acc, i32x4 a, i32x4 b) {                                        \
+    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));                                              \
+  }                                                                                                                     \
+  /* acc (VGPRs) += a b */                                                                                              \
+  static __device__ __forceinline__ void v_acc(f32x16& acc, i32x4 a, i32x4 b) {                                         \
+    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));                                              \
+  }                                                                                                                     \
+  /* the same with the B operand in AGPRs */                                                                            \
+  static __device__ __forceinline__ void v_init_ba(f32x16& acc, i32x4 a, i32x4 b) {                                     \
+    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));                                              \
+  }                                                                                                                     \
+  static __device__ __forceinline__ void v_acc_ba(f32x16& acc, i32x4 a, i32x4 b) {                                      \
+    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));                                              \
+  }                                                                                                                     \
+  /* acc (AGPRs) += a b */                                                                                              \
+  static __device__ __forceinline__ void a_acc(f32x16& acc, i32x4 a, i32x4 b) {                                         \
+    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));                                              \
   }
-  __builtin_amdgcn_sched_barrier(0);
+#else
+#define FO_MFMA_BODY(MNEMONIC)                                                                                          \
+  static __device__ __forceinline__ void v_init(f32x16&, i32x4, i32x4) {}                                               \
+  static __device__ __forceinline__ void v_acc(f32x16&, i32x4, i32x4) {}                                                \
+  static __device__ __forceinline__ void v_init_ba(f32x16&, i32x4, i32x4) {}                                            \
+  static __device__ __forceinline__ void v_acc_ba(f32x16&, i32x4, i32x4) {}                                             \
+  static __device__ __forceinline__ void a_acc(f32x16&, i32x4, i32x4) {}
+#endif
+template <> struct AsmMfma<__bf16> { FO_MFMA_BODY("v_mfma_f32_32x32x16_bf16") };
+template <> struct AsmMfma<_Float16> { FO_MFMA_BODY("v_mfma_f32_32x32x16_f16") };
+#undef FO_MFMA_BODY
+
+// Wait states for an MFMA result to become readable by VALU instructions the compiler places (see above). The values
+// to be read are passed through empty volatile statements after the wait, so that no read can be moved above it.
+template <int N>
+__device__ __forceinline__ void mfma_result_fence_a(f32x16 (&acc)[N]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+a"(acc[i]));
+#endif
+}
+template <int N>
+__device__ __forceinline__ void mfma_result_fence_v(f32x16 (&acc)[N]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(acc[i]));
+#endif
+}
+// x *= a for an accumulator that lives in AGPRs, element by element in place through one VGPR (left to the compiler,
+// every accumulator moves to VGPRs at once, at the cost of the whole kernel's register budget)
+__device__ __forceinline__ void scale_acc(f32x16& acc, float a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float e = acc[r], tmp;
+    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1" : "+a"(e), "=&v"(tmp) : "v"(a));
+    acc[r] = e;
+  }
+#endif
 }
 
-template <typename T, int D, bool CAUSAL, int SCHED, int NG>
-__global__ void __launch_bounds__(kPipeBM / (32 * NG) * 64) attn_fwd_pipe_kernel(const AttnParams prm) {
-  constexpr int NWAVES = kPipeBM / (32 * NG);     // 8 waves x 32 rows, or 4 waves x 64 rows (two row groups per wave)
-  typedef typename Ops<T>::vec8 vec8;
+template <typename T, int D, bool CAUSAL, int QB, int DBG>
+__global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel(const AttnParams prm) {
+  constexpr int kWideWaves = kWideBM / (32 * QB);
+  typedef __attribute__((ext_vector_type(2))) T vec2;
   constexpr int ROW_BYTES = D * 2;
-  constexpr int CHUNKS = ROW_BYTES / 16;
   constexpr int TILE_BYTES = kBN * ROW_BYTES;
-  constexpr int KSTEPS = D / 16;                 // MFMAs of one sub-tile's Q K^T
+  constexpr int HALF_BYTES = TILE_BYTES / 2;     // one 32-key sub-tile
+  constexpr int KSTEPS = D / 16;                 // K fragments of one sub-tile; each feeds QB MFMAs (one per 32-row query block)
   constexpr int DBLK = D / 32;
-  constexpr int NB = KSTEPS / 4;                 // batches (of 4 MFMAs) per phase: 2 at D = 128, 1 at D = 64
-  constexpr int DMA_PER_WAVE = TILE_BYTES / 1024 / NWAVES;
-  constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;
-  static_assert(2 * DBLK == KSTEPS && DMA_PER_WAVE >= 1, "tile shape");
+  constexpr int VFRAGS = 2 * DBLK;               // V^T fragments of one sub-tile (2 steps of 16 keys x D/32 blocks)
+  constexpr int BLOCKS = TILE_BYTES / 1024;      // 1 KiB copy blocks per tile
+  constexpr int DMA_PER_WAVE = BLOCKS / kWideWaves;
+  static_assert(VFRAGS == KSTEPS && DMA_PER_WAVE >= 1 && KSTEPS >= 4, "tile shape");
 
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   FO_LDS char* smem = (FO_LDS char*)smem_raw;    // K ring (kRing tiles) | V ring (kRing tiles)
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
-  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int wave_s = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hh = lane >> 5;
-  const int L16 = lane & 15;
-  const int g16 = (lane >> 4) & 1;
 
   const int n_bh = prm.B * prm.H;
   int bh, qblk;
@@ -429,8 +493,8 @@ __global__ void __launch_bounds__(kPipeBM / (32 * NG) * 64) attn_fwd_pipe_kernel
     }
   }
   const int b = bh / prm.H, h = bh % prm.H;
-  const int q0 = qblk * kPipeBM;
-  const int q0w = q0 + wave_s * 32 * NG;
+  const int q0 = qblk * kWideBM;
+  const int q0w = q0 + wave_s * 32 * QB;
   const int Sq = prm.Sq, Sk = prm.Sk;
   const T* __restrict__ qbase = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
   const T* __restrict__ kbase = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1];
@@ -438,320 +502,362 @@ __global__ void __launch_bounds__(kPipeBM / (32 * NG) * 64) attn_fwd_pipe_kernel
 
   int n_tiles, n_w;                       // tiles the workgroup walks / tiles in which this wave has unmasked keys
   if constexpr (CAUSAL) {
-    n_tiles = (min(Sk, q0 + kPipeBM) + kBN - 1) / kBN;
-    n_w = min(n_tiles, (q0w + 32 * NG - 1) / kBN + 1);
+    n_tiles = (min(Sk, q0 + kWideBM) + kBN - 1) / kBN;
+    n_w = min(n_tiles, (q0w + 32 * QB - 1) / kBN + 1);
   } else {
     n_tiles = (Sk + kBN - 1) / kBN;
     n_w = n_tiles;
   }
 
-  // ---- global -> LDS copies
-  uint32_t k_off[DMA_PER_WAVE], v_off[DMA_PER_WAVE];
-#pragma unroll
-  for (int i = 0; i < DMA_PER_WAVE; ++i) {
-    const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane / CHUNKS;
-    const int col = ((lane % CHUNKS) ^ swz<D>(row)) * 8;
-    k_off[i] = (uint32_t)(row * (int)prm.ks[2] + col) * 2u;
-    v_off[i] = (uint32_t)(row * (int)prm.vs[2] + col) * 2u;
-  }
+  // ---- LDS layout of a tile: 1 KiB blocks, each written by ONE direct-to-LDS instruction (64 lanes x 16 bytes, lane
+  // order) and laid out so that every fragment read of the inner loop is "lane base + compile-time offset" over
+  // consecutive addresses - no swizzle arithmetic, no bank conflicts, one address register per matrix.
+  //   K tile: block (hf, kp, r16) = rows 32 hf + 16 r16 .. +15 of the tile, 64 bytes (k-steps 2kp, 2kp+1) of each row,
+  //     at ((hf * D/32 + kp) * 2 + r16) KiB; inside, the 16-byte piece (k-step 2kp + kk, half hh, row rr) sits at
+  //     kk*512 + hh*256 + rr*16. The A-operand read of k-step ks (lane = row l32, half hh) is then
+  //     (l32/16)*1024 + hh*256 + (l32%16)*16  +  hf*HALF_BYTES + (ks/2)*2048 + (ks%2)*512.
+  //   V tile: block (hf, t, db) = rows 32 hf + 16 t .. +15, 64 bytes (d = 32 db .. +31) of each row, at
+  //     (hf * D/16 + t * D/32 + db) KiB; inside, the two transposing reads (rows +0..7 / +8..15) each get 512
+  //     consecutive bytes in the lane order of that read: lane*8  +  hf*HALF_BYTES + (t*D/32 + db)*1024 + half*512.
+  // Which 16 bytes of global memory a copy lane fetches follows from that; per row the four lanes that fetch from it
+  // cover 64 consecutive bytes.
+  const int k_lane_row = lane & 15, k_lane_col = (lane >> 4) * 8;
+  const int v_m = lane & 31;
+  const int v_lane_row = 8 * (lane >> 5) + 4 * (v_m >> 4) + ((v_m & 7) >> 1), v_lane_col = 16 * ((v_m >> 3) & 1) + 8 * (v_m & 1);
+  const uint32_t k_off = (uint32_t)(k_lane_row * (int)prm.ks[2] + k_lane_col) * 2u;
+  const uint32_t v_off = (uint32_t)(v_lane_row * (int)prm.vs[2] + v_lane_col) * 2u;
   // one tile of K (ring 0) or V (ring 1) into slot tile % kRing
-  auto issue = [&](const T* base, int64_t stride, const uint32_t* off, int tile, int ring) {
+  auto issue = [&](auto is_v, int tile) {
+    constexpr bool V = decltype(is_v)::value;
+    const T* base = V ? vbase : kbase;
+    const int64_t stride = V ? prm.vs[2] : prm.ks[2];
     const int key0 = tile * kBN;
-    FO_LDS char* dst = smem + (kRing * ring + (tile & (kRing - 1))) * TILE_BYTES;
-    if (key0 + kBN <= Sk) {
-      const char* src = (const char*)(base + (int64_t)key0 * stride);
+    FO_LDS char* dst = smem + (kRing * (V ? 1 : 0) + (tile & (kRing - 1))) * TILE_BYTES;
 #pragma unroll
-      for (int i = 0; i < DMA_PER_WAVE; ++i) dma16_uniform_base(src, off[i], dst + (wave_s * DMA_PER_WAVE + i) * 1024);
-    } else {
-      int lane_here = lane;                            // (opaque: keeps this rare path's address math inside it)
-      asm volatile("" : "+v"(lane_here));
-#pragma unroll
-      for (int i = 0; i < DMA_PER_WAVE; ++i) {
-        const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane_here / CHUNKS;
-        const int col = ((lane_here % CHUNKS) ^ swz<D>(row)) * 8;
-        const int key = min(key0 + row, Sk - 1);       // rows past the end re-read the last key (masked later)
-        dma16_lane_ptr(base + (int64_t)key * stride + col, dst + (wave_s * DMA_PER_WAVE + i) * 1024);
+    for (int i = 0; i < DMA_PER_WAVE; ++i) {
+      const int blk = wave_s * DMA_PER_WAVE + i;
+      const int hf = blk / (BLOCKS / 2), in_half = blk % (BLOCKS / 2);
+      // first row (in the tile) and first column of the block
+      const int row0 = V ? 32 * hf + 16 * (in_half / DBLK) : 32 * hf + 16 * (in_half & 1);
+      const int col0 = V ? 32 * (in_half % DBLK) : 32 * (in_half >> 1);
+      if (key0 + kBN <= Sk) {
+        const char* src = (const char*)(base + (int64_t)(key0 + row0) * stride + col0);
+        dma16_uniform_base(src, V ? v_off : k_off, dst + blk * 1024);
+      } else {
+        int lane_here = lane;                            // (opaque: keeps this rare path's address math inside it)
+        asm volatile("" : "+v"(lane_here));
+        const int m = lane_here & 31;
+        const int lrow = V ? 8 * (lane_here >> 5) + 4 * (m >> 4) + ((m & 7) >> 1) : (lane_here & 15);
+        const int lcol = V ? 16 * ((m >> 3) & 1) + 8 * (m & 1) : (lane_here >> 4) * 8;
+        const int key = min(key0 + row0 + lrow, Sk - 1);   // rows past the end re-read the last key (masked later)
+        dma16_lane_ptr(base + (int64_t)key * stride + col0 + lcol, dst + blk * 1024);
       }
     }
   };
   // batch(t), issued at the top of tile t: K(t+3) and V(t+2). Returns the number of copies this lane issued.
   auto issue_batch = [&](int t) -> int {
     int n = 0;
-    if (t + 3 < n_tiles && t + 3 >= 0) { issue(kbase, prm.ks[2], k_off, t + 3, 0); n += DMA_PER_WAVE; }
-    if (t + 2 < n_tiles && t + 2 >= 0) { issue(vbase, prm.vs[2], v_off, t + 2, 1); n += DMA_PER_WAVE; }
+    if (t + 3 < n_tiles && t + 3 >= 0) { issue(std::false_type{}, t + 3); n += DMA_PER_WAVE; }
+    if (t + 2 < n_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2); n += DMA_PER_WAVE; }
     return n;
   };
   issue_batch(-3);
   issue_batch(-2);
   int last_batch = issue_batch(-1);
 
-  // ---- Q^T fragments (B operand of S^T = K Q^T)
-  vec8 qf[NG][KSTEPS];
+  // ---- Q^T fragments (B operand of S^T = K Q^T), QB blocks of 32 query rows
+  i32x4 qf[QB][KSTEPS];
 #pragma unroll
-  for (int g = 0; g < NG; ++g) {
-    const int qrow = min(q0w + 32 * g + l32, Sq - 1);
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qrow = min(q0w + 32 * qb + l32, Sq - 1);
     const T* qp = qbase + (int64_t)qrow * prm.qs[2] + 8 * hh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[g][ks] = *(const vec8*)(qp + 16 * ks);
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[qb][ks] = *(const i32x4*)(qp + 16 * ks);
   }
 #pragma unroll
-  for (int g = 0; g < NG; ++g)
+  for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[g][ks]));   // wait for Q here, never inside the loop
+    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" : "+a"(qf[qb][ks]));   // wait for Q here, never inside the loop; held in AGPRs
 
-  f32x16 oacc[NG][DBLK];
+  f32x16 oacc[DBLK][QB];       // O^T accumulators (AGPRs): d-block x query block
 #pragma unroll
-  for (int g = 0; g < NG; ++g)
+  for (int i = 0; i < DBLK; ++i)
 #pragma unroll
-    for (int i = 0; i < DBLK; ++i)
+    for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[g][i][r] = 0.0f;
-  f32x16 Sacc[NG];             // scores of the sub-tile being produced (MFMA accumulators)
-  f32x16 sv[NG];               // scores of the sub-tile being consumed: copied out of Sacc, masked
-  vec8 pf[NG][2];              // P of the sub-tile being multiplied with V (two 16-key steps)
-  vec8 FB[2][4];               // LDS fragment batches: current and next (each fragment feeds NG MFMAs)
-  float m_run[NG], l_run[NG], mloc[NG];
+      for (int r = 0; r < 16; ++r) oacc[i][qb][r] = 0.0f;
+  f32x16 S[2][QB];             // scores: sub-tile s, query block qb live in S[s & 1][qb]
+  i32x4 PF[2][QB][2];          // P of sub-tile s: PF[s & 1][qb][16-key step]
+  constexpr int RD = QB == 2 ? 4 : 2;       // must divide the number of fragments of a sub-tile
+  static_assert(KSTEPS % RD == 0, "fragment ring");
+  i32x4 KF[RD], VF[RD];        // LDS fragment rings, refilled RD fragments ahead of use
+  float m_run[QB], l_run[QB];
 #pragma unroll
-  for (int g = 0; g < NG; ++g) { m_run[g] = -INFINITY; l_run[g] = 0.0f; mloc[g] = -INFINITY; }
+  for (int qb = 0; qb < QB; ++qb) { m_run[qb] = -INFINITY; l_run[qb] = 0.0f; }
   const float c = prm.scale_log2e;
 
-  // Held in registers for the whole kernel: 8 byte offsets for K (one per k-step) and 2 x DBLK for V^T; everything else
-  // about a fragment address (ring slot, sub-tile half, 16-key step) is a wave-uniform or compile-time addend.
-  uint32_t koffs[KSTEPS], voffs0[DBLK], voffs1[DBLK];
-  {
-    const int ksw = swz<D>(l32);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) koffs[ks] = (uint32_t)(l32 * ROW_BYTES + (((2 * ks + hh) ^ ksw) * 16));
-    const int vrow0 = 4 * hh + (L16 >> 2);
-    const int vsw0 = swz<D>(vrow0), vsw1 = swz<D>(vrow0 + 8);
-    const int vsub = (L16 & 1) * 8;
-    const int vchunk = 2 * g16 + ((L16 & 3) >> 1);
-#pragma unroll
-    for (int db = 0; db < DBLK; ++db) {
-      voffs0[db] = (uint32_t)(vrow0 * ROW_BYTES + vsub + (((4 * db + vchunk) ^ vsw0) * 16));
-      voffs1[db] = (uint32_t)((vrow0 + 8) * ROW_BYTES + vsub + (((4 * db + vchunk) ^ vsw1) * 16));
-    }
-  }
-  auto read_k4 = [&](vec8 (&dst)[4], FO_LDS const char* kt, int hf, int ks0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) dst[i] = *(FO_LDS const vec8*)(kt + hf * 32 * ROW_BYTES + koffs[ks0 + i]);
+  const uint32_t k_lane = (uint32_t)((l32 >> 4) * 1024 + hh * 256 + (l32 & 15) * 16);
+  const uint32_t v_lane = (uint32_t)(kRing * TILE_BYTES + lane * 8);
+  // byte offset of sub-tile `sub` (tile sub/2, half sub%2) inside its ring
+  auto sub_base = [&](int sub) -> uint32_t { return (uint32_t)(((sub >> 1) & (kRing - 1)) * TILE_BYTES + (sub & 1) * HALF_BYTES); };
+  // K fragment ks / V^T fragment idx (16-key step idx / DBLK, d-block idx % DBLK) of the sub-tile whose base
+  // (lane part included) is `base`. A sub-tile index past the end reads a valid but meaningless ring slot; such
+  // fragments are never used.
+  auto k_frag = [&](uint32_t base, int ks) -> i32x4 {
+    return *(FO_LDS const i32x4*)(smem + base + (ks >> 1) * 2048 + (ks & 1) * 512);
   };
-  // four V^T fragments: batch bi of sub-tile half hf. At D = 128: t = 2*hf + bi, db = 0..3. At D = 64: t = 2*hf + i/2, db = i%2.
-  auto read_v4 = [&](vec8 (&dst)[4], FO_LDS const char* vt, int hf, int bi) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int t = (DBLK == 4) ? 2 * hf + bi : 2 * hf + (i >> 1);
-      const int db = (DBLK == 4) ? i : (i & 1);
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(vt + 16 * t * ROW_BYTES + voffs0[db]));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(vt + 16 * t * ROW_BYTES + voffs1[db]));
-      dst[i] = __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
-  };
-  auto k_slot = [&](int tile) -> FO_LDS const char* { return smem + (tile & (kRing - 1)) * TILE_BYTES; };
-  auto v_slot = [&](int tile) -> FO_LDS const char* { return smem + (kRing + (tile & (kRing - 1))) * TILE_BYTES; };
-
-  // ---- VALU pieces
-  // exponentials of elements [e0, e1) of sv -> pf, psum
-  auto exp_part = [&](const float (&mc)[NG], float (&psum)[NG], int e0, int e1) {
-#pragma unroll
-    for (int g = 0; g < NG; ++g)
-#pragma unroll
-      for (int e = e0; e < e1; ++e) {
-        const float x = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[g][e], c, -mc[g]));
-        psum[g] += x;                              // summed in fp32 before rounding (flash_attention_triton.py:203)
-        pf[g][e >> 3][e & 7] = (T)x;               // rounded to the operand type for P.V (:237)
-      }
-  };
-  // elements [e0, e1) of the sub-tile just produced (half hf of tile): copy out of the accumulators, mask, fold into the
-  // row max. The mask is applied unconditionally (two VALU operations per element, hidden behind phase B's MFMAs): a
-  // branch on "this tile needs a mask" would split the straight-line block that the MFMA/VALU interleave relies on.
-  // Register r holds key key_base + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); it is dead iff key > q or key >= Sk,
-  // i.e. iff lim + koff(r) > 0 with lim = max(key_base - q, key_base - Sk + 1).
-  auto max_part = [&](int tile, int hf, int e0, int e1) {
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-      const int key_base = tile * kBN + 32 * hf + 4 * hh;
-      int lim = key_base - Sk + 1;
-      if (CAUSAL) lim = max(lim, key_base - (q0w + 32 * g + l32));
-#pragma unroll
-      for (int r = e0; r < e1; ++r) sv[g][r] = (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : Sacc[g][r];
-#pragma unroll
-      for (int r = e0; r < e1; r += 2) mloc[g] = fmaxf(fmaxf(mloc[g], sv[g][r]), sv[g][r + 1]);
-    }
-  };
-  // finish the row max, raise the reference maximum where needed (lazily), rescale O and l
-  auto settle = [&]() {
-    bool raise = false;
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-      mloc[g] = fmaxf(mloc[g], half_swap(mloc[g]));
-      raise = raise || (mloc[g] * c > m_run[g] * c + kLazyLog2);
-    }
-    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-#pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        const float m_new = fmaxf(m_run[g], mloc[g]);    // finite from the first sub-tile on: key 0 is never masked
-        const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * c);
-        m_run[g] = m_new;
-        l_run[g] *= alpha;
-#pragma unroll
-        for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[g][i][r] *= alpha;
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < NG; ++g) mloc[g] = -INFINITY;
+  auto v_frag = [&](uint32_t base, int idx) -> i32x4 {
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(smem + base + idx * 1024));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(smem + base + idx * 1024 + 512));
+    return __builtin_bit_cast(i32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  // ---- one full step. On entry FB[0] holds the first K batch of sub-tile (tq, hq).
-  //   phase A: Sacc = K(tq, hq) Q^T       ||  P = exp2(sv c - m c)                 (sv = sub-tile (te, he), the previous one)
-  //   phase B: O += V(te, he)^T P^T       ||  sv = mask(Sacc), row max
-  //   then settle; on exit FB[0] holds the first K batch of the sub-tile after (tq, hq) (garbage past the end: unused).
-  auto full_step = [&](int tq, int hq, int te, int he) {
-    FO_LDS const char* kt = k_slot(tq);
-    FO_LDS const char* vt = v_slot(te);
-    FO_LDS const char* kt_next = hq ? k_slot(tq + 1) : kt;
-    float mc[NG], psum[NG];
+  // ---- one pipeline step for sub-tile s (parity P = s & 1), as micro-groups of one MFMA each:
+  //   HAS_QK: S[P^1] = K(s+1) Q^T;   HAS_PV: O += V(s-1)^T PF[P^1]^T;   always: S[P] -> PF[P] = exp2(S c - m c), row sums.
+  // On entry KF holds K fragments 0..RD-1 of sub-tile s+1 and VF holds V^T fragments 0..RD-1 of sub-tile s-1; on exit
+  // the same for the next step.
+  //
+  // The reference m of the exponentials is not the running row maximum but a stale one: the micro-groups compute no
+  // maximum at all. P may therefore exceed 1; as long as it stays below 2^12 the fp32 accumulators and the
+  // half-precision P lose no relative precision, and O / l and LSE = m + log(l) do not depend on the reference. At
+  // the end of the step the row sums tell whether some P got large (or overflowed: the first step starts from
+  // m = -inf); only then (rarely) the step's P is recomputed from the still intact scores against the true maximum,
+  // and O and l are rescaled. The result is that of the exact recurrence (flash_attention_triton.py:200-213,241-243)
+  // up to rounding.
+  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked) {
+    constexpr int P = decltype(parity)::value;
+    constexpr bool HAS_QK = decltype(has_qk)::value, HAS_PV = decltype(has_pv)::value, MASK = decltype(masked)::value;
+    constexpr int NM = QB * KSTEPS;                                     // MFMAs of one kind
+    constexpr int G = (HAS_QK ? NM : 0) + (HAS_PV ? NM : 0);            // micro-groups
+    constexpr int NEL = 16 * QB;                                        // scores per lane
+    // Group 0 only issues its MFMA: the scores of this sub-tile were written by MFMAs up to the last-but-one group of
+    // the previous step. Then the mask (if any), then the exponentials.
+    constexpr int GMASK = 1;
+    constexpr int GE0 = MASK ? 2 : 1, NE = G - GE0;                     // groups that carry the exponentials
+    // (an opaque copy of the sub-tile index: the variants of this step are selected by branches, and identical address
+    // arithmetic in two branches would otherwise be hoisted above them, out of its micro-group)
+    int s = s_in;
+    asm volatile("" : "+s"(s));
+    const uint32_t kb1 = k_lane + sub_base(s + 1), kb2 = k_lane + sub_base(s + 2);
+    const uint32_t vb0 = v_lane + sub_base(s - 1), vb1 = v_lane + sub_base(s);
+    float mc[QB], psum[QB];
 #pragma unroll
-    for (int g = 0; g < NG; ++g) {
-      mc[g] = m_run[g] * c;
-      psum[g] = 0.0f;
+    for (int b2 = 0; b2 < QB; ++b2) { mc[b2] = m_run[b2] * c; psum[b2] = 0.0f; }
+    float ex[NEL];
+    // score e of NEL: query block, accumulator register (the first 8 registers of every block first: they are the
+    // first 16-key step of P V)
+    auto el_qb = [](int e) { return QB == 2 ? (e >> 3) & 1 : 0; };
+    auto el_reg = [](int e) { return QB == 2 ? 8 * (e >> 4) + (e & 7) : e; };
 #pragma unroll
-      for (int r = 0; r < 16; ++r) Sacc[g][r] = 0.0f;
-    }
-    // phase A
-#pragma unroll
-    for (int bi = 0; bi < NB; ++bi) {
-      if (bi + 1 < NB) read_k4(FB[(bi + 1) & 1], kt, hq, 4 * (bi + 1));
-      else read_v4(FB[(bi + 1) & 1], vt, he, 0);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int g = 0; g < NG; ++g) Sacc[g] = Ops<T>::mfma(FB[bi & 1][i], qf[g][4 * bi + i], Sacc[g]);
-      exp_part(mc, psum, bi * (16 / NB), (bi + 1) * (16 / NB));
-      if (bi + 1 < NB) sched_batch<SCHED != 0, NG, 4, (16 / NB) * 5 / 8 + 1, (16 / NB) / 4>();
-      else sched_batch<SCHED != 0, NG, 8, (16 / NB) * 5 / 8 + 1, (16 / NB) / 4>();
-    }
-#pragma unroll
-    for (int g = 0; g < NG; ++g) l_run[g] += psum[g];
-    // phase B (fragment buffers continue to alternate: batch NB of this step sits in FB[NB & 1])
-#pragma unroll
-    for (int bi = 0; bi < NB; ++bi) {
-      const int cur = (NB + bi) & 1;
-      if (bi + 1 < NB) read_v4(FB[cur ^ 1], vt, he, bi + 1);
-      else read_k4(FB[cur ^ 1], kt_next, hq ^ 1, 0);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int t = (DBLK == 4) ? bi : (i >> 1);       // 16-key step inside the sub-tile
-        const int db = (DBLK == 4) ? i : (i & 1);
-#pragma unroll
-        for (int g = 0; g < NG; ++g) oacc[g][db] = Ops<T>::mfma(FB[cur][i], pf[g][t], oacc[g][db]);
+    for (int g = 0; g < G; ++g) {
+      // -- the MFMA of this micro-group, and the LDS read that refills a fragment once every query block has used it
+      const bool is_qk = HAS_QK && (!HAS_PV || (g & 1) == 0);
+      const int i = (HAS_QK && HAS_PV) ? (g >> 1) : g;                 // index among the MFMAs of its kind
+      const int f = i / QB, qb = i % QB;                               // fragment, query block
+      if (DBG & 8) asm volatile("s_nop 1");
+      if (is_qk) {
+        if (f == 0) AsmMfma<T>::v_init_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
+        else AsmMfma<T>::v_acc_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
+        if (qb == QB - 1 && !(DBG & 4)) KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb1, f + RD) : k_frag(kb2, f + RD - KSTEPS);
+      } else {
+        AsmMfma<T>::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[P ^ 1][qb][f / DBLK]);
+        if (qb == QB - 1 && !(DBG & 4)) VF[f % RD] = (f + RD < VFRAGS) ? v_frag(vb0, f + RD) : v_frag(vb1, f + RD - VFRAGS);
       }
-      max_part(tq, hq, bi * (16 / NB), (bi + 1) * (16 / NB));
-      if (bi + 1 < NB) sched_batch<SCHED != 0, NG, 8, (16 / NB) * 5 / 8 + 1, 0>();
-      else sched_batch<SCHED != 0, NG, 4, (16 / NB) * 5 / 8 + 1, 0>();
-    }
-    settle();
-  };
-  static_assert(NB == 2 || NB == 1, "fragment buffer parity below assumes one or two batches per phase");
-
-  // ---- first sub-tile alone: Sacc = K(0, 0) Q^T, copy out, mask, max, settle; leaves the next K batch in FB[0]
-  auto first_step = [&]() {
-    FO_LDS const char* kt = k_slot(0);
-    read_k4(FB[0], kt, 0, 0);
+      if constexpr (!HAS_PV) {
+        if (g < RD) VF[g] = v_frag(vb1, g);   // first step: the next one expects the first V^T fragments of sub-tile s
+      }
+      // -- this group's share of the softmax arithmetic
+      if (MASK && g == GMASK) {
+        // register r holds key key_base + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); dead iff key > q or key >= Sk,
+        // i.e. iff lim + koff(r) > 0 with lim = max(key_base - q, key_base - Sk + 1)
+        const int key_base = s * 32 + 4 * hh;
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+        for (int b2 = 0; b2 < QB; ++b2) {
+          int lim = key_base - Sk + 1;
+          if (CAUSAL) lim = max(lim, key_base - (q0w + 32 * b2 + l32));
 #pragma unroll
-      for (int r = 0; r < 16; ++r) Sacc[g][r] = 0.0f;
+          for (int r = 0; r < 16; ++r) S[P][b2][r] = (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : S[P][b2][r];
+        }
+      }
+      if (g >= GE0) {
 #pragma unroll
-    for (int bi = 0; bi < NB; ++bi) {
-      if (bi + 1 < NB) read_k4(FB[(bi + 1) & 1], kt, 0, 4 * (bi + 1));
+        for (int e = 0; e < NEL; ++e)
+          if (GE0 + (e * NE) / NEL == g) {
+            const int b2 = el_qb(e), r = el_reg(e);
+            ex[e] = (DBG & 2) ? S[P][b2][r] : __builtin_amdgcn_exp2f(__builtin_fmaf(S[P][b2][r], c, -mc[b2]));
+            psum[b2] += ex[e];                                         // summed in fp32 before rounding (flash_attention_triton.py:203)
+            asm volatile("" ::"v"(ex[e]), "v"(psum[b2]));              // a use inside the micro-group: keeps the compiler from sinking this work out of it
+          }
+        // A pair is rounded to the operand type for P.V (flash_attention_triton.py:237) one group after its second
+        // element (the last group finishes what is left).
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int g = 0; g < NG; ++g) Sacc[g] = Ops<T>::mfma(FB[bi & 1][i], qf[g][4 * bi + i], Sacc[g]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    read_k4(FB[0], kt, 1, 0);
-    max_part(0, 0, 0, 16);
-    settle();
-  };
-  // ---- last sub-tile (te, he) of this wave alone: P = exp2(sv ...), O += V^T P^T
-  auto last_step = [&](int te, int he) {
-    FO_LDS const char* vt = v_slot(te);
-    float mc[NG], psum[NG];
-#pragma unroll
-    for (int g = 0; g < NG; ++g) { mc[g] = m_run[g] * c; psum[g] = 0.0f; }
-    read_v4(FB[0], vt, he, 0);
-    exp_part(mc, psum, 0, 16);
-#pragma unroll
-    for (int g = 0; g < NG; ++g) l_run[g] += psum[g];
-#pragma unroll
-    for (int bi = 0; bi < NB; ++bi) {
-      if (bi + 1 < NB) read_v4(FB[(bi + 1) & 1], vt, he, bi + 1);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int t = (DBLK == 4) ? bi : (i >> 1);
-        const int db = (DBLK == 4) ? i : (i & 1);
-#pragma unroll
-        for (int g = 0; g < NG; ++g) oacc[g][db] = Ops<T>::mfma(FB[bi & 1][i], pf[g][t], oacc[g][db]);
+        for (int pr = 0; pr < NEL / 2; ++pr) {
+          const int ready = GE0 + ((2 * pr + 1) * NE) / NEL + 1;
+          if ((ready < G ? ready : G - 1) == g) {
+            const int e = 2 * pr, b2 = el_qb(e), r = el_reg(e);
+            const vec2 pk = {(T)ex[e], (T)ex[e + 1]};
+            const int pki = __builtin_bit_cast(int, pk);
+            asm volatile("" ::"v"(pki));
+            PF[P][b2][r >> 3][(r & 7) >> 1] = pki;
+          }
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    // -- end of step: did some P get large (or infinite, or NaN from a masked score against m = -inf)?
+    bool redo = false;
+#pragma unroll
+    for (int b2 = 0; b2 < QB; ++b2) redo = redo || !(psum[b2] <= kLargeRowSum);
+    if (__builtin_amdgcn_ballot_w64(redo) != 0 && !(DBG & 2)) {
+      // rare: true row maxima of this sub-tile, new references, P and row sums again, O and l rescaled
+#pragma unroll
+      for (int d = 0; d < DBLK; ++d) mfma_result_fence_a(oacc[d]);
+#pragma unroll
+      for (int b2 = 0; b2 < QB; ++b2) {
+        float mloc = S[P][b2][0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, S[P][b2][r]);
+        mloc = fmaxf(mloc, half_swap(mloc));
+        const float m_new = fmaxf(m_run[b2], mloc);                    // finite from the first sub-tile on: key 0 is never masked
+        const float alpha = __builtin_amdgcn_exp2f((m_run[b2] - m_new) * c);
+        const float mcn = m_new * c;
+        float ps = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[P][b2][r], c, -mcn));
+          const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[P][b2][r + 1], c, -mcn));
+          ps += p0;
+          ps += p1;
+          const vec2 pk = {(T)p0, (T)p1};
+          PF[P][b2][r >> 3][(r & 7) >> 1] = __builtin_bit_cast(int, pk);
+        }
+        psum[b2] = ps;
+        m_run[b2] = m_new;
+        l_run[b2] *= alpha;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int d = 0; d < DBLK; ++d) scale_acc(oacc[d][b2], alpha);
+      }
+    }
+#pragma unroll
+    for (int b2 = 0; b2 < QB; ++b2) l_run[b2] += psum[b2];
   };
+  using std::integral_constant;
+  typedef integral_constant<int, 0> P0;
+  typedef integral_constant<int, 1> P1;
+  typedef std::true_type Y;
+  typedef std::false_type N;
 
-  // ---- tile loop. Iteration j: [S(j,0) || P(j-1,1)] [PV(j-1,1) || max(j,0)] [S(j,1) || P(j,0)] [PV(j,0) || max(j,1)]
-  // reads K(j), V(j-1), V(j). Batches up to (j-2) must have landed: K(j+1) and V(j) among them.
-  for (int j = 0; j < n_tiles; ++j) {
+  // ---- tile loop. Tile j runs the steps of sub-tiles 2j and 2j+1; they read K(j), K(j+1), V(j-1), V(j).
+  // At its top, copy batches up to (j-2) must have landed - K(j+1) and V(j) are among them - while batch (j-1) may still
+  // be in flight; after the barrier every wave is done with tile j-1, so batch j may overwrite K(j-1) and V(j-2).
+  auto tile_top = [&](int j) {
     if (last_batch >= 2 * DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
     else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    last_batch = issue_batch(j);
-    if (j < n_w) {
-      if (j == 0) first_step();
-      else full_step(j, 0, j - 1, 1);
-      full_step(j, 1, j, 0);
-    } else if (j == n_w) {
-      last_step(j - 1, 1);
+    last_batch = (DBG & 1) ? 0 : issue_batch(j);
+  };
+  // Tiles that need the mask (causal diagonal, keys past the end) are a suffix of the wave's tiles. The hot loops are
+  // kept free of alternatives: unmasked tiles, then masked tiles, then the last tile, whose second step has no scores
+  // left to compute; the first and last tiles always take the masking variant.
+  int j_mask = n_w;                                   // first tile that needs the mask
+  if (CAUSAL) j_mask = min(j_mask, (q0w + 1) / kBN);   // smallest j with 64 j + 63 > q0w
+  if (Sk % kBN != 0) j_mask = min(j_mask, n_tiles - 1);
+
+  // first tile: fill the pipeline - S(0) on its own, then a step that has nothing to multiply yet
+  tile_top(0);
+  {
+    const uint32_t kb0 = k_lane + sub_base(0), kb1 = k_lane + sub_base(1);
+#pragma unroll
+    for (int i = 0; i < RD; ++i) KF[i] = k_frag(kb0, i);
+#pragma unroll
+    for (int f = 0; f < KSTEPS; ++f) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        if (f == 0) AsmMfma<T>::v_init_ba(S[0][qb], KF[f % RD], qf[qb][f]);
+        else AsmMfma<T>::v_acc_ba(S[0][qb], KF[f % RD], qf[qb][f]);
+      }
+      KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb0, f + RD) : k_frag(kb1, f + RD - KSTEPS);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
-  if (n_w == n_tiles) last_step(n_tiles - 1, 1);
+  mfma_result_fence_v(S[0]);
+  step(0, P0{}, Y{}, N{}, Y{});
+  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}); else step(1, P1{}, N{}, Y{}, Y{});
+  // The steps above may have parked a few registers in scratch memory. Wait here, visibly to the compiler, for any
+  // reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0) wait that executes on
+  // every iteration and also drains the copies in flight, which it does not see.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), nothing else
+  int j = 1;
+  for (; j < min(j_mask, n_w - 1); ++j) {
+    tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, N{});
+    step(2 * j + 1, P1{}, Y{}, Y{}, N{});
+  }
+  for (; j < n_w - 1; ++j) {
+    tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, Y{});
+    step(2 * j + 1, P1{}, Y{}, Y{}, Y{});
+  }
+  if (j < n_w) {
+    tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, Y{});
+    step(2 * j + 1, P1{}, N{}, Y{}, Y{});
+    ++j;
+  }
+  {
+    // drain: O += V(last)^T P(last)^T for this wave's last sub-tile (2*n_w - 1, odd parity); VF holds its first fragments
+    const uint32_t vbl = v_lane + sub_base(2 * n_w - 1);
+#pragma unroll
+    for (int f = 0; f < VFRAGS; ++f) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) AsmMfma<T>::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[1][qb][f / DBLK]);
+      if (f + RD < VFRAGS) VF[f % RD] = v_frag(vbl, f + RD);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // tiles in which this wave has nothing to do (causal): keep feeding the workgroup's rings
+  for (; j < n_tiles; ++j) tile_top(j);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: normalise, write O and LSE
 #pragma unroll
-  for (int g = 0; g < NG; ++g) {
-    const float l_tot = l_run[g] + half_swap(l_run[g]);
+  for (int d = 0; d < DBLK; ++d) mfma_result_fence_a(oacc[d]);
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const float l_tot = l_run[qb] + half_swap(l_run[qb]);
     const float inv = 1.0f / l_tot;
-    const int qi = q0w + 32 * g + l32;
-    if (qi < Sq) {
-      T* op = (T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)qi * prm.os[2];
+    const int qi = q0w + 32 * qb + l32;
+    T* op = (T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)min(qi, Sq - 1) * prm.os[2];
 #pragma unroll
-      for (int db = 0; db < DBLK; ++db)
+    for (int db = 0; db < DBLK; ++db) {
+      f32x16 t = oacc[db][qb];
+      asm volatile("" : "+v"(t));                       // one accumulator at a time through VGPRs
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          typedef __attribute__((ext_vector_type(4))) T vec4;
-          vec4 o4;
+      for (int rg = 0; rg < 4; ++rg) {
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        vec4 o4;
 #pragma unroll
-          for (int u = 0; u < 4; ++u) o4[u] = (T)(oacc[g][db][rg * 4 + u] * inv);
-          *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
-        }
-      if (prm.lse != nullptr && hh == 0)
-        prm.lse[(int64_t)bh * Sq + qi] = (m_run[g] * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+        for (int u = 0; u < 4; ++u) o4[u] = (T)(t[rg * 4 + u] * inv);
+        if (qi < Sq) *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
+    if (qi < Sq && prm.lse != nullptr && hh == 0)
+      prm.lse[(int64_t)bh * Sq + qi] = (m_run[qb] * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   }
 }
 
-template <typename T, int D, bool CAUSAL, int SCHED, int NG>
-static int launch_pipe(AttnParams p, hipStream_t stream) {
+template <typename T, int D, bool CAUSAL, int QB, int DBG = 0>
+static int launch_wide(AttnParams p, hipStream_t stream) {
   const size_t lds = 2 * (size_t)kRing * kBN * D * 2;
-  p.n_qblk = (p.Sq + kPipeBM - 1) / kPipeBM;
+  p.n_qblk = (p.Sq + kWideBM - 1) / kWideBM;
   const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_pipe_kernel<T, D, CAUSAL, SCHED, NG>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
-  attn_fwd_pipe_kernel<T, D, CAUSAL, SCHED, NG><<<grid, kPipeBM / (32 * NG) * 64, lds, stream>>>(p);
+  attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG><<<grid, kWideBM / (32 * QB) * 64, lds, stream>>>(p);
   return launch_status();
 }
 
@@ -771,10 +877,25 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
   const int v = g_attn_variant < 0 ? 0 : g_attn_variant;
-  if (v == 16) return causal ? launch_pipe<T, D, true, 0, 1>(p, stream) : launch_pipe<T, D, false, 0, 1>(p, stream);
-  if (v == 17) return causal ? launch_pipe<T, D, true, 1, 1>(p, stream) : launch_pipe<T, D, false, 1, 1>(p, stream);
-  if (v == 18) return causal ? launch_pipe<T, D, true, 0, 2>(p, stream) : launch_pipe<T, D, false, 0, 2>(p, stream);
-  if (v == 19) return causal ? launch_pipe<T, D, true, 1, 2>(p, stream) : launch_pipe<T, D, false, 1, 2>(p, stream);
+  if constexpr (D == 128) {
+    // 16: eight waves x 32 rows; 32: four waves x 64 rows. 17..31 / 33..47: timing ablations of those two (non-causal
+    // only, WRONG results): bit 0 no global->LDS copies, bit 1 no exponentials, bit 2 no LDS fragment reads, bit 3 two
+    // idle cycles before every MFMA.
+    if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
+    if (v == 32) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
+    if (v > 16 && v < 48 && !causal) {
+      switch (v) {
+        case 17: return launch_wide<T, D, false, 1, 1>(p, stream);
+        case 18: return launch_wide<T, D, false, 1, 2>(p, stream);
+        case 20: return launch_wide<T, D, false, 1, 4>(p, stream);
+        case 23: return launch_wide<T, D, false, 1, 7>(p, stream);
+        case 24: return launch_wide<T, D, false, 1, 8>(p, stream);
+        case 39: return launch_wide<T, D, false, 2, 7>(p, stream);
+        case 40: return launch_wide<T, D, false, 2, 8>(p, stream);
+        default: return FO_ERR_UNSUPPORTED;
+      }
+    }
+  }
   if (D == 128 && causal && sizeof(T) == 2) {
     switch (v >> 1) {
       case 1: return launch_one<T, D, true, true, 1>(p, stream);
