@@ -1,0 +1,156 @@
+"""Checks the gfx950 assembly of kernels that issue MFMAs as inline assembly for the two data hazards that the
+compiler's hazard recognizer handles for its own MFMA instructions but cannot see inside an asm statement:
+
+  1. an MFMA source register (A, B or C, VGPR or AGPR) written by a VALU instruction needs 2 wait states before the
+     MFMA reads it (measured on MI355X: back-to-back gives wrong products; v_accvgpr_read counts as VALU);
+  2. a register written by an 8-pass MFMA (32x32x16 f16/bf16) needs 11 wait states before any other instruction than
+     an MFMA touches it.
+
+A wait state is one issued instruction (s_nop N counts N+1). For rule 2 time is modelled in wait states; an MFMA is
+taken to issue no earlier than 8 wait states after the previous one (the matrix pipe is busy for its 8 passes), every
+other instruction advances time by one. Control flow is treated conservatively for rule 1 (an MFMA within two
+instructions after a label fails) and in layout order for rule 2 (the kernels fence every out-of-line reader
+explicitly).
+
+Used by build.py: the attention kernels are first compiled without wait states in front of their MFMAs; if this
+check reports anything, they are compiled again with them.
+"""
+from __future__ import annotations
+
+import re
+from typing import Iterable, List, Set, Tuple
+
+_REG = re.compile(r"\b([va])(\d+)\b|\b([va])\[(\d+):(\d+)\]")
+
+
+def _regs(operand: str) -> Set[Tuple[str, int]]:
+    out = set()
+    for m in _REG.finditer(operand):
+        if m.group(1):
+            out.add((m.group(1), int(m.group(2))))
+        else:
+            out.update((m.group(3), i) for i in range(int(m.group(4)), int(m.group(5)) + 1))
+    return out
+
+
+def _split_operands(rest: str) -> List[str]:
+    ops, depth, cur = [], 0, ""
+    for ch in rest:
+        if ch == "[":
+            depth += 1
+        elif ch == "]":
+            depth -= 1
+        if ch == "," and depth == 0:
+            ops.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        ops.append(cur.strip())
+    return ops
+
+
+# VALU instructions that write more than their first operand
+_SWAPS = ("v_permlane32_swap", "v_permlane16_swap", "v_swap_b32")
+MFMA_PASSES = 8
+VALU_TO_MFMA = 2          # wait states between a VALU write and an MFMA read
+MFMA_TO_OTHER = 11        # wait states between an 8-pass MFMA write and any non-MFMA access
+
+
+def lint_function(lines: Iterable[str], name: str) -> List[str]:
+    problems: List[str] = []
+    recent: List[Set[Tuple[str, int]]] = []     # registers written by VALU in each of the last instructions (newest last)
+    since_label = 10**9
+    t = 0                                         # time in wait states
+    last_mfma_issue = -10**9
+    ready = {}                                    # register -> time from which a non-MFMA instruction may touch it
+    for ln, raw in enumerate(lines, 1):
+        line = raw.split(";")[0].strip()
+        if not line or line.startswith("."):
+            if line.startswith(".LBB") or (line.endswith(":") and not line.startswith(".")):
+                since_label = 0
+                recent = []
+            continue
+        if line.endswith(":"):
+            since_label = 0
+            recent = []
+            continue
+        parts = line.split(None, 1)
+        op = parts[0]
+        ops = _split_operands(parts[1]) if len(parts) > 1 else []
+        if op.startswith("v_mfma") or op.startswith("v_smfmac"):
+            srcs = set()
+            for o in ops[1:]:
+                srcs |= _regs(o)
+            if since_label < VALU_TO_MFMA:
+                problems.append(f"{name}:{ln}: MFMA {since_label} instruction(s) after a label: {line}")
+            for age, written in enumerate(reversed(recent[-VALU_TO_MFMA:])):
+                hit = srcs & written
+                if hit:
+                    problems.append(f"{name}:{ln}: MFMA reads {sorted(hit)[:4]} written by a VALU instruction {age} wait state(s) earlier: {line}")
+            issue = max(t, last_mfma_issue + MFMA_PASSES)
+            last_mfma_issue = issue
+            for r in _regs(ops[0]):
+                ready[r] = issue + MFMA_TO_OTHER + 1
+            t = issue + 1
+            recent.append(set())
+            since_label += 1
+            continue
+        # any other instruction: rule 2 on every register it names
+        touched = set()
+        for o in ops:
+            touched |= _regs(o)
+        for r in touched:
+            if ready.get(r, -1) > t:
+                problems.append(f"{name}:{ln}: {r[0]}{r[1]} touched {ready[r] - t} wait state(s) too early after an MFMA wrote it: {line}")
+                break
+        for r in touched:
+            ready.pop(r, None)
+        written = set()
+        if op.startswith("v_") and ops:
+            written |= _regs(ops[0])
+            if op.startswith(_SWAPS) and len(ops) > 1:
+                written |= _regs(ops[1])
+        states = 1
+        if op == "s_nop" and ops:
+            try:
+                states = int(ops[0], 0) + 1
+            except ValueError:
+                states = 1
+        for _ in range(states):
+            recent.append(set())
+        recent[-1] = written
+        if len(recent) > 8:
+            recent = recent[-8:]
+        t += states
+        since_label += states
+    return problems
+
+
+def lint_file(path: str, name_filter: str) -> List[str]:
+    """Lints every function of the assembly file whose symbol matches the regular expression `name_filter`."""
+    pat = re.compile(name_filter)
+    problems: List[str] = []
+    cur_name, cur_lines = None, []
+    with open(path) as f:
+        for raw in f:
+            s = raw.rstrip("\n")
+            if cur_name is None:
+                head = s.split(";")[0].rstrip()
+                if head.endswith(":") and not head.startswith((".", " ", "\t")) and pat.search(head):
+                    cur_name, cur_lines = head[:-1], []
+            else:
+                if s.startswith(".Lfunc_end"):
+                    problems += lint_function(cur_lines, cur_name)
+                    cur_name = None
+                else:
+                    cur_lines.append(s)
+    return problems
+
+
+if __name__ == "__main__":
+    import sys
+    found = lint_file(sys.argv[1], sys.argv[2] if len(sys.argv) > 2 else "attn_fwd_wide_kernel")
+    for p in found[:50]:
+        print(p)
+    print(f"{len(found)} problem(s)")

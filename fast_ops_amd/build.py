@@ -39,6 +39,9 @@ SOURCES = {
     # would silently leave them rolled, with their register arrays in scratch memory.
     "attn_fwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
 }
+# sources whose generated assembly is checked by asm_lint: source -> regular expression of the kernel symbols to check
+# (the instantiations with a non-zero last template argument are timing experiments with wrong results by design)
+ASM_LINTED = {"attn_fwd.hip": r"attn_fwd_wide_kernel.*ELi0EEEvNS_10AttnParamsE"}
 
 
 def _hipcc() -> str:
@@ -54,21 +57,44 @@ def _newest_header_mtime() -> float:
     return max(os.path.getmtime(p) for p in paths if os.path.exists(p))
 
 
+def _run_hipcc(cmd: list, src: str, verbose: bool) -> None:
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass does not know the device-only target feature and says so; everything else is shown
+    err = "\n".join(l for l in res.stderr.splitlines() if "is not a recognized feature for this target" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+    if err.strip() and verbose:
+        print(err, file=sys.stderr)
+
+
 def _compile_one(hipcc: str, src: str, extra: list, force: bool, verbose: bool) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    stem = os.path.splitext(src)[0]
+    obj = os.path.join(OBJ_DIR, stem + ".o")
     src_path = os.path.join(CSRC, src)
     stale = force or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(src_path), _newest_header_mtime())
-    if stale:
-        cmd = [hipcc] + COMMON_FLAGS + extra + ["-c", src_path, "-o", obj]
+    if not stale:
+        return obj
+    if src not in ASM_LINTED:
+        _run_hipcc([hipcc] + COMMON_FLAGS + extra + ["-c", src_path, "-o", obj], src, verbose)
+        return obj
+    # Kernels with inline-assembly MFMAs: first without wait states in front of the MFMAs of the inner loops, keeping
+    # the device assembly, which is then checked for the hazards the compiler cannot see inside an asm statement. If the
+    # check finds one, compile again with the wait states.
+    from .asm_lint import lint_file
+    _run_hipcc([hipcc] + COMMON_FLAGS + extra + ["-DFO_MFMA_NOPS=0", "-save-temps=obj", "-c", src_path, "-o", obj], src, verbose)
+    asm = os.path.join(OBJ_DIR, f"{stem}-hip-amdgcn-amd-amdhsa-{ARCH}.s")
+    problems = lint_file(asm, ASM_LINTED[src]) if os.path.exists(asm) else [f"{asm} was not produced"]
+    for f in os.listdir(OBJ_DIR):           # the other intermediate files are large and of no further use
+        if f.startswith(stem + "-") or f.startswith(stem + ".hip-"):
+            os.remove(os.path.join(OBJ_DIR, f))
+    if problems:
         if verbose:
-            print(" ".join(cmd), flush=True)
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        # the host pass does not know the device-only target feature and says so; everything else is shown
-        err = "\n".join(l for l in res.stderr.splitlines() if "is not a recognized feature for this target" not in l)
-        if res.returncode != 0:
-            raise RuntimeError(f"hipcc failed for {src}:\n{err}")
-        if err.strip() and verbose:
-            print(err, file=sys.stderr)
+            print(f"{src}: {len(problems)} MFMA hazard(s) without wait states, e.g. {problems[0]}\n  -> compiling with wait states", flush=True)
+        _run_hipcc([hipcc] + COMMON_FLAGS + extra + ["-DFO_MFMA_NOPS=1", "-c", src_path, "-o", obj], src, verbose)
+    elif verbose:
+        print(f"{src}: inline-assembly MFMAs checked, no hazard", flush=True)
     return obj
 
 

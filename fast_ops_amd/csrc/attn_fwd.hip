@@ -392,38 +392,37 @@ constexpr float kLargeRowSum = 4096.0f;   // a lane's 16-key row sum above this 
 
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 
-template <typename T> struct AsmMfma;
+// NOP: two wait states in front of the MFMA (see above). FO_MFMA_NOPS = 1 puts them in front of every MFMA; with 0
+// the MFMAs inside the tile loops go without, which is only correct if no VALU write of a source lands within two
+// instructions before them: the build checks the generated assembly for that and falls back to 1 if it finds one.
+#ifndef FO_MFMA_NOPS
+#define FO_MFMA_NOPS 1
+#endif
+template <typename T, bool NOP> struct AsmMfma;
 #if defined(__HIP_DEVICE_COMPILE__)
-#define FO_MFMA_BODY(MNEMONIC)                                                                                          \
-  /* acc (VGPRs) = a b */                                                                                               \
-  static __device__ __forceinline__ void v_init(f32x16& acc, i32x4 a, i32x4 b) {                                        \
-    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));                                              \
-  }                                                                                                                     \
-  /* acc (VGPRs) += a b */                                                                                              \
-  static __device__ __forceinline__ void v_acc(f32x16& acc, i32x4 a, i32x4 b) {                                         \
-    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));                                              \
-  }                                                                                                                     \
-  /* the same with the B operand in AGPRs */                                                                            \
+#define FO_MFMA_BODY(PRE, MNEMONIC)                                                                                     \
+  /* acc (VGPRs) = a b, B operand in AGPRs */                                                                           \
   static __device__ __forceinline__ void v_init_ba(f32x16& acc, i32x4 a, i32x4 b) {                                     \
-    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));                                              \
+    asm volatile(PRE MNEMONIC " %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));                                          \
   }                                                                                                                     \
+  /* acc (VGPRs) += a b, B operand in AGPRs */                                                                          \
   static __device__ __forceinline__ void v_acc_ba(f32x16& acc, i32x4 a, i32x4 b) {                                      \
-    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));                                              \
+    asm volatile(PRE MNEMONIC " %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));                                          \
   }                                                                                                                     \
   /* acc (AGPRs) += a b */                                                                                              \
   static __device__ __forceinline__ void a_acc(f32x16& acc, i32x4 a, i32x4 b) {                                         \
-    asm volatile("s_nop 1\n\t" MNEMONIC " %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));                                              \
+    asm volatile(PRE MNEMONIC " %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));                                          \
   }
 #else
-#define FO_MFMA_BODY(MNEMONIC)                                                                                          \
-  static __device__ __forceinline__ void v_init(f32x16&, i32x4, i32x4) {}                                               \
-  static __device__ __forceinline__ void v_acc(f32x16&, i32x4, i32x4) {}                                                \
+#define FO_MFMA_BODY(PRE, MNEMONIC)                                                                                     \
   static __device__ __forceinline__ void v_init_ba(f32x16&, i32x4, i32x4) {}                                            \
   static __device__ __forceinline__ void v_acc_ba(f32x16&, i32x4, i32x4) {}                                             \
   static __device__ __forceinline__ void a_acc(f32x16&, i32x4, i32x4) {}
 #endif
-template <> struct AsmMfma<__bf16> { FO_MFMA_BODY("v_mfma_f32_32x32x16_bf16") };
-template <> struct AsmMfma<_Float16> { FO_MFMA_BODY("v_mfma_f32_32x32x16_f16") };
+template <> struct AsmMfma<__bf16, true> { FO_MFMA_BODY("s_nop 1\n\t", "v_mfma_f32_32x32x16_bf16") };
+template <> struct AsmMfma<_Float16, true> { FO_MFMA_BODY("s_nop 1\n\t", "v_mfma_f32_32x32x16_f16") };
+template <> struct AsmMfma<__bf16, false> { FO_MFMA_BODY("", "v_mfma_f32_32x32x16_bf16") };
+template <> struct AsmMfma<_Float16, false> { FO_MFMA_BODY("", "v_mfma_f32_32x32x16_f16") };
 #undef FO_MFMA_BODY
 
 // Wait states for an MFMA result to become readable by VALU instructions the compiler places (see above). The values
@@ -460,6 +459,7 @@ __device__ __forceinline__ void scale_acc(f32x16& acc, float a) {
 template <typename T, int D, bool CAUSAL, int QB, int DBG>
 __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel(const AttnParams prm) {
   constexpr int kWideWaves = kWideBM / (32 * QB);
+  typedef AsmMfma<T, true> Mfma;                  // outside the loops: always with wait states
   typedef __attribute__((ext_vector_type(2))) T vec2;
   constexpr int ROW_BYTES = D * 2;
   constexpr int TILE_BYTES = kBN * ROW_BYTES;
@@ -624,7 +624,9 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // m = -inf); only then (rarely) the step's P is recomputed from the still intact scores against the true maximum,
   // and O and l are rescaled. The result is that of the exact recurrence (flash_attention_triton.py:200-213,241-243)
   // up to rounding.
-  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked) {
+  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop) {
+    // inside the loops the MFMAs go without wait states in front unless the build asked for them (see above)
+    typedef AsmMfma<T, !(decltype(in_loop)::value && !FO_MFMA_NOPS)> Mfma;
     constexpr int P = decltype(parity)::value;
     constexpr bool HAS_QK = decltype(has_qk)::value, HAS_PV = decltype(has_pv)::value, MASK = decltype(masked)::value;
     constexpr int NM = QB * KSTEPS;                                     // MFMAs of one kind
@@ -654,13 +656,12 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       const bool is_qk = HAS_QK && (!HAS_PV || (g & 1) == 0);
       const int i = (HAS_QK && HAS_PV) ? (g >> 1) : g;                 // index among the MFMAs of its kind
       const int f = i / QB, qb = i % QB;                               // fragment, query block
-      if (DBG & 8) asm volatile("s_nop 1");
       if (is_qk) {
-        if (f == 0) AsmMfma<T>::v_init_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
-        else AsmMfma<T>::v_acc_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
+        if (f == 0) Mfma::v_init_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
+        else Mfma::v_acc_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
         if (qb == QB - 1 && !(DBG & 4)) KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb1, f + RD) : k_frag(kb2, f + RD - KSTEPS);
       } else {
-        AsmMfma<T>::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[P ^ 1][qb][f / DBLK]);
+        Mfma::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[P ^ 1][qb][f / DBLK]);
         if (qb == QB - 1 && !(DBG & 4)) VF[f % RD] = (f + RD < VFRAGS) ? v_frag(vb0, f + RD) : v_frag(vb1, f + RD - VFRAGS);
       }
       if constexpr (!HAS_PV) {
@@ -752,10 +753,16 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // At its top, copy batches up to (j-2) must have landed - K(j+1) and V(j) are among them - while batch (j-1) may still
   // be in flight; after the barrier every wave is done with tile j-1, so batch j may overwrite K(j-1) and V(j-2).
   auto tile_top = [&](int j) {
-    if (last_batch >= 2 * DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
-    else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    if (!(DBG & 32)) {
+      if (last_batch >= 2 * DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
+      else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    // A bare barrier: __syncthreads() would first wait for every LDS read in flight, i.e. drain the fragment rings once
+    // per tile. Nothing needs that wait: the reads in flight here target K(j) and V(j-1), not the slots batch j
+    // overwrites, and copies are made visible by the vmcnt wait above (it covers this wave's own pieces; the barrier
+    // extends that to everyone's).
+    if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
     last_batch = (DBG & 1) ? 0 : issue_batch(j);
   };
   // Tiles that need the mask (causal diagonal, keys past the end) are a suffix of the wave's tiles. The hot loops are
@@ -775,16 +782,16 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     for (int f = 0; f < KSTEPS; ++f) {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
-        if (f == 0) AsmMfma<T>::v_init_ba(S[0][qb], KF[f % RD], qf[qb][f]);
-        else AsmMfma<T>::v_acc_ba(S[0][qb], KF[f % RD], qf[qb][f]);
+        if (f == 0) Mfma::v_init_ba(S[0][qb], KF[f % RD], qf[qb][f]);
+        else Mfma::v_acc_ba(S[0][qb], KF[f % RD], qf[qb][f]);
       }
       KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb0, f + RD) : k_frag(kb1, f + RD - KSTEPS);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   mfma_result_fence_v(S[0]);
-  step(0, P0{}, Y{}, N{}, Y{});
-  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}); else step(1, P1{}, N{}, Y{}, Y{});
+  step(0, P0{}, Y{}, N{}, Y{}, N{});
+  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}); else step(1, P1{}, N{}, Y{}, Y{}, N{});
   // The steps above may have parked a few registers in scratch memory. Wait here, visibly to the compiler, for any
   // reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0) wait that executes on
   // every iteration and also drains the copies in flight, which it does not see.
@@ -792,18 +799,18 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   int j = 1;
   for (; j < min(j_mask, n_w - 1); ++j) {
     tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, N{});
-    step(2 * j + 1, P1{}, Y{}, Y{}, N{});
+    step(2 * j, P0{}, Y{}, Y{}, N{}, Y{});
+    step(2 * j + 1, P1{}, Y{}, Y{}, N{}, Y{});
   }
   for (; j < n_w - 1; ++j) {
     tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, Y{});
-    step(2 * j + 1, P1{}, Y{}, Y{}, Y{});
+    step(2 * j, P0{}, Y{}, Y{}, Y{}, Y{});
+    step(2 * j + 1, P1{}, Y{}, Y{}, Y{}, Y{});
   }
   if (j < n_w) {
     tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, Y{});
-    step(2 * j + 1, P1{}, N{}, Y{}, Y{});
+    step(2 * j, P0{}, Y{}, Y{}, Y{}, N{});
+    step(2 * j + 1, P1{}, N{}, Y{}, Y{}, N{});
     ++j;
   }
   {
@@ -812,7 +819,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
 #pragma unroll
     for (int f = 0; f < VFRAGS; ++f) {
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) AsmMfma<T>::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[1][qb][f / DBLK]);
+      for (int qb = 0; qb < QB; ++qb) Mfma::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[1][qb][f / DBLK]);
       if (f + RD < VFRAGS) VF[f % RD] = v_frag(vbl, f + RD);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -883,15 +890,23 @@ static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
     // idle cycles before every MFMA.
     if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
     if (v == 32) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
-    if (v > 16 && v < 48 && !causal) {
+    // timing ablations (WRONG results), non-causal only: 256 + bits for eight waves, 512 + bits for four.
+    // bit 0 no global->LDS copies, 1 no exponentials, 2 no LDS fragment reads,
+    // 5 no wait for copies, 6 no barrier
+    if constexpr (std::is_same<T, __bf16>::value) if (v >= 256 && !causal) {
       switch (v) {
-        case 17: return launch_wide<T, D, false, 1, 1>(p, stream);
-        case 18: return launch_wide<T, D, false, 1, 2>(p, stream);
-        case 20: return launch_wide<T, D, false, 1, 4>(p, stream);
-        case 23: return launch_wide<T, D, false, 1, 7>(p, stream);
-        case 24: return launch_wide<T, D, false, 1, 8>(p, stream);
-        case 39: return launch_wide<T, D, false, 2, 7>(p, stream);
-        case 40: return launch_wide<T, D, false, 2, 8>(p, stream);
+        case 256 + 1: return launch_wide<T, D, false, 1, 1>(p, stream);
+        case 256 + 2: return launch_wide<T, D, false, 1, 2>(p, stream);
+        case 256 + 4: return launch_wide<T, D, false, 1, 4>(p, stream);
+        case 256 + 7: return launch_wide<T, D, false, 1, 7>(p, stream);
+        case 256 + 32: return launch_wide<T, D, false, 1, 32>(p, stream);
+        case 256 + 64: return launch_wide<T, D, false, 1, 64>(p, stream);
+        case 512 + 1: return launch_wide<T, D, false, 2, 1>(p, stream);
+        case 512 + 2: return launch_wide<T, D, false, 2, 2>(p, stream);
+        case 512 + 4: return launch_wide<T, D, false, 2, 4>(p, stream);
+        case 512 + 32: return launch_wide<T, D, false, 2, 32>(p, stream);
+        case 512 + 64: return launch_wide<T, D, false, 2, 64>(p, stream);
+        case 512 + 7: return launch_wide<T, D, false, 2, 7>(p, stream);
         default: return FO_ERR_UNSUPPORTED;
       }
     }
