@@ -456,6 +456,9 @@ __device__ __forceinline__ void scale_acc(f32x16& acc, float a) {
 #endif
 }
 
+// workgroups per head of the wide kernel
+__host__ __device__ inline int wide_items(int n_qblk, bool causal) { return causal ? (n_qblk + 1) / 2 : n_qblk; }
+
 template <typename T, int D, bool CAUSAL, int QB, int DBG>
 __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel(const AttnParams prm) {
   constexpr int kWideWaves = kWideBM / (32 * QB);
@@ -479,20 +482,31 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   const int l32 = lane & 31;
   const int hh = lane >> 5;
 
+  // A causal workgroup takes two query blocks, one after the other: block n-1-i (the heaviest left) and block i, so
+  // that every workgroup has the same amount of work (n+1 tiles' worth) whatever i is. Non-causal: one block each.
   const int n_bh = prm.B * prm.H;
-  int bh, qblk;
+  const int n_items = wide_items(prm.n_qblk, CAUSAL);
+  int bh, item;
   {
     const int id = blockIdx.x;
     if ((n_bh & 7) == 0) {
-      const int x = id & 7, j = id >> 3;
-      bh = x + 8 * (j / prm.n_qblk);
-      qblk = prm.n_qblk - 1 - (j % prm.n_qblk);
+      const int x = id & 7, j = id >> 3;          // XCD, position in that XCD's list: one head after the other
+      bh = x + 8 * (j / n_items);
+      item = j % n_items;
     } else {
       bh = id % n_bh;
-      qblk = prm.n_qblk - 1 - id / n_bh;
+      item = id / n_bh;
     }
   }
   const int b = bh / prm.H, h = bh % prm.H;
+  const int n_pass = (CAUSAL && prm.n_qblk - 1 - item != item) ? 2 : 1;
+  for (int pass = 0; pass < n_pass; ++pass) {
+  const int qblk = CAUSAL ? (pass == 0 ? prm.n_qblk - 1 - item : item) : item;
+  if (pass > 0) {
+    // the other waves may still be reading the rings, and this wave's stores of O still count as memory operations in flight
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
   const int q0 = qblk * kWideBM;
   const int q0w = q0 + wave_s * 32 * QB;
   const int Sq = prm.Sq, Sk = prm.Sk;
@@ -854,13 +868,14 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     if (qi < Sq && prm.lse != nullptr && hh == 0)
       prm.lse[(int64_t)bh * Sq + qi] = (m_run[qb] * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   }
+  }   // pass
 }
 
 template <typename T, int D, bool CAUSAL, int QB, int DBG = 0>
 static int launch_wide(AttnParams p, hipStream_t stream) {
   const size_t lds = 2 * (size_t)kRing * kBN * D * 2;
   p.n_qblk = (p.Sq + kWideBM - 1) / kWideBM;
-  const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
+  const unsigned grid = (unsigned)(wide_items(p.n_qblk, CAUSAL) * p.B * p.H);
   static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
@@ -883,11 +898,10 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 // WRONG results (bit 1: keep re-using the first tiles instead of copying new ones; bit 2: no exponentials).
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
-  const int v = g_attn_variant < 0 ? 0 : g_attn_variant;
+  // default: the wide kernel (four waves x 64 rows) for head_dim 128, the 128-row kernel for head_dim 64
+  const int v = g_attn_variant < 0 ? (D == 128 ? 32 : 0) : g_attn_variant;
   if constexpr (D == 128) {
-    // 16: eight waves x 32 rows; 32: four waves x 64 rows. 17..31 / 33..47: timing ablations of those two (non-causal
-    // only, WRONG results): bit 0 no global->LDS copies, bit 1 no exponentials, bit 2 no LDS fragment reads, bit 3 two
-    // idle cycles before every MFMA.
+    // 16: wide kernel, eight waves x 32 rows; 32: wide kernel, four waves x 64 rows
     if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
     if (v == 32) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
     // timing ablations (WRONG results), non-causal only: 256 + bits for eight waves, 512 + bits for four.

@@ -84,6 +84,39 @@ def test_ragged_and_unequal_lengths(shape, causal, D):
     _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype):
+    # head_dim 128 works on 256-row query blocks (two per workgroup when causal) and a four-slot ring of key tiles
+    B, H, Sq, Sk = shape
+    _run_and_check(B, H, Sq, Sk, 128, dtype, causal, seed=Sq + Sk)
+
+
+@pytest.mark.parametrize("pattern", ["growing", "shrinking", "spikes"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+def test_moving_row_maximum(pattern, causal, D, dtype):
+    # scores whose row maximum keeps moving (or sits far above the rest) exercise the rescaling of the running
+    # softmax state: keys scaled so that scaled scores span tens of units
+    B, H, Sq, Sk = 1, 2, 384, 640
+    q, k, v = _qkv(B, H, Sq, Sk, D, torch.float32, seed=7)
+    pos = torch.arange(Sk, dtype=torch.float32)
+    if pattern == "growing":
+        gain = 0.5 + 6.0 * pos / Sk
+    elif pattern == "shrinking":
+        gain = 6.5 - 6.0 * pos / Sk
+    else:
+        gain = torch.where(pos % 97 == 5, torch.tensor(12.0), torch.tensor(1.0))
+    k = k * gain[None, None, :, None]
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal)
+    o, lse = multi_head_attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal, return_lse=True)
+    torch.cuda.synchronize()
+    _check(o, lse, o_ref, lse_ref, f"{pattern} D{D} {dtype} causal={causal}")
+
+
 def test_golden_fixture():
     z = np.load(GOLDEN)
     to16 = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16)
