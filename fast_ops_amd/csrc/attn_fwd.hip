@@ -568,8 +568,32 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       }
     }
   };
+  // The common case, both tiles complete: this wave's blocks have fixed places inside a tile (pointers for tile 0
+  // are loop-invariant scalars), and the tile's distance from tile 0 is added to the per-lane offset.
+  const char* k_src0[DMA_PER_WAVE];
+  const char* v_src0[DMA_PER_WAVE];
+#pragma unroll
+  for (int i = 0; i < DMA_PER_WAVE; ++i) {
+    const int blk = wave_s * DMA_PER_WAVE + i;
+    const int hf = blk / (BLOCKS / 2), in_half = blk % (BLOCKS / 2);
+    k_src0[i] = (const char*)(kbase + (int64_t)(32 * hf + 16 * (in_half & 1)) * prm.ks[2] + 32 * (in_half >> 1));
+    v_src0[i] = (const char*)(vbase + (int64_t)(32 * hf + 16 * (in_half / DBLK)) * prm.vs[2] + 32 * (in_half % DBLK));
+  }
+  const uint32_t k_tile_bytes = (uint32_t)(kBN * (int)prm.ks[2]) * 2u, v_tile_bytes = (uint32_t)(kBN * (int)prm.vs[2]) * 2u;
+  const int n_full = min(n_tiles, Sk / kBN);          // tiles below this one are complete
   // batch(t), issued at the top of tile t: K(t+3) and V(t+2). Returns the number of copies this lane issued.
   auto issue_batch = [&](int t) -> int {
+    if (t + 3 < n_full && t + 2 >= 0) {
+      const uint32_t ko = k_off + (uint32_t)(t + 3) * k_tile_bytes, vo = v_off + (uint32_t)(t + 2) * v_tile_bytes;
+      FO_LDS char* kdst = smem + ((t + 3) & (kRing - 1)) * TILE_BYTES + wave_s * DMA_PER_WAVE * 1024;
+      FO_LDS char* vdst = smem + (kRing + ((t + 2) & (kRing - 1))) * TILE_BYTES + wave_s * DMA_PER_WAVE * 1024;
+#pragma unroll
+      for (int i = 0; i < DMA_PER_WAVE; ++i) {
+        dma16_uniform_base(k_src0[i], ko, kdst + i * 1024);
+        dma16_uniform_base(v_src0[i], vo, vdst + i * 1024);
+      }
+      return 2 * DMA_PER_WAVE;
+    }
     int n = 0;
     if (t + 3 < n_tiles && t + 3 >= 0) { issue(std::false_type{}, t + 3); n += DMA_PER_WAVE; }
     if (t + 2 < n_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2); n += DMA_PER_WAVE; }
@@ -649,7 +673,9 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     // Group 0 only issues its MFMA: the scores of this sub-tile were written by MFMAs up to the last-but-one group of
     // the previous step. Then the mask (if any), then the exponentials.
     constexpr int GMASK = 1;
-    constexpr int GE0 = MASK ? 2 : 1, NE = G - GE0;                     // groups that carry the exponentials
+    constexpr int GE0 = MASK ? 2 : 1;                                   // first group that may read the scores
+    constexpr int NE = G - 2 - GE0;                                     // groups GE0+1 .. G-2 carry the exponentials
+    static_assert(NE >= 2, "too few micro-groups");
     // (an opaque copy of the sub-tile index: the variants of this step are selected by branches, and identical address
     // arithmetic in two branches would otherwise be hoisted above them, out of its micro-group)
     int s = s_in;
@@ -694,25 +720,28 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
           for (int r = 0; r < 16; ++r) S[P][b2][r] = (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : S[P][b2][r];
         }
       }
-      if (g >= GE0) {
+      // Three stages, one micro-group apart, so that no instruction of a group waits for another one of the same
+      // group: scale-and-shift of score e in group GE(e) - 1, its exponential in GE(e), the row sum and (for a finished
+      // pair) the rounding to the operand type for P.V (flash_attention_triton.py:237) in GE(e) + 1.
 #pragma unroll
-        for (int e = 0; e < NEL; ++e)
-          if (GE0 + (e * NE) / NEL == g) {
-            const int b2 = el_qb(e), r = el_reg(e);
-            ex[e] = (DBG & 2) ? S[P][b2][r] : __builtin_amdgcn_exp2f(__builtin_fmaf(S[P][b2][r], c, -mc[b2]));
-            psum[b2] += ex[e];                                         // summed in fp32 before rounding (flash_attention_triton.py:203)
-            asm volatile("" ::"v"(ex[e]), "v"(psum[b2]));              // a use inside the micro-group: keeps the compiler from sinking this work out of it
-          }
-        // A pair is rounded to the operand type for P.V (flash_attention_triton.py:237) one group after its second
-        // element (the last group finishes what is left).
-#pragma unroll
-        for (int pr = 0; pr < NEL / 2; ++pr) {
-          const int ready = GE0 + ((2 * pr + 1) * NE) / NEL + 1;
-          if ((ready < G ? ready : G - 1) == g) {
-            const int e = 2 * pr, b2 = el_qb(e), r = el_reg(e);
-            const vec2 pk = {(T)ex[e], (T)ex[e + 1]};
-            const int pki = __builtin_bit_cast(int, pk);
-            asm volatile("" ::"v"(pki));
+      for (int e = 0; e < NEL; ++e) {
+        const int ge = GE0 + 1 + (e * NE) / NEL;
+        const int b2 = el_qb(e), r = el_reg(e);
+        if (ge - 1 == g) {
+          ex[e] = (DBG & 2) ? S[P][b2][r] : __builtin_fmaf(S[P][b2][r], c, -mc[b2]);
+          asm volatile("" : "+v"(ex[e]));                              // pins the instruction to this micro-group
+        }
+        if (ge == g) {
+          if (!(DBG & 2)) ex[e] = __builtin_amdgcn_exp2f(ex[e]);
+          asm volatile("" : "+v"(ex[e]));
+        }
+        if (ge + 1 == g) {
+          psum[b2] += ex[e];                                           // summed in fp32 before rounding (flash_attention_triton.py:203)
+          asm volatile("" : "+v"(psum[b2]));
+          if (e & 1) {
+            const vec2 pk = {(T)ex[e - 1], (T)ex[e]};
+            int pki = __builtin_bit_cast(int, pk);
+            asm volatile("" : "+v"(pki));
             PF[P][b2][r >> 3][(r & 7) >> 1] = pki;
           }
         }
@@ -768,7 +797,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // be in flight; after the barrier every wave is done with tile j-1, so batch j may overwrite K(j-1) and V(j-2).
   auto tile_top = [&](int j) {
     if (!(DBG & 32)) {
-      if (last_batch >= 2 * DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
+      if (__builtin_expect(last_batch == 2 * DMA_PER_WAVE, 1)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
       else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
       else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
@@ -898,8 +927,15 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 // WRONG results (bit 1: keep re-using the first tiles instead of copying new ones; bit 2: no exponentials).
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
-  // default: the wide kernel (four waves x 64 rows) for head_dim 128, the 128-row kernel for head_dim 64
-  const int v = g_attn_variant < 0 ? (D == 128 ? 32 : 0) : g_attn_variant;
+  // default: the wide kernel (eight waves x 32 rows) for head_dim 128, the 128-row kernel for head_dim 64
+  // (the wide kernel addresses a head's keys with 32-bit byte offsets)
+  // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
+  // 128-row kernel, with four times as many workgroups, fills the chip better
+  static const int n_cu = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256; return n; }();
+  const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
+  const bool wide_ok = D == 128 && (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
+  int v = g_attn_variant < 0 ? (wide_ok && wide_wgs >= n_cu ? 16 : 0) : g_attn_variant;
+  if (!wide_ok && v >= 16) v = 0;
   if constexpr (D == 128) {
     // 16: wide kernel, eight waves x 32 rows; 32: wide kernel, four waves x 64 rows
     if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
