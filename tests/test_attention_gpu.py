@@ -11,6 +11,7 @@ import pytest
 import torch
 
 from fast_ops.flash_attention.flash_attention import FlashAttentionFunction, flash_attn, multi_head_attention
+from fast_ops_amd import _lib
 from oracle.attention_oracle import attention_fwd_oracle
 
 pytestmark = pytest.mark.gpu
@@ -37,6 +38,18 @@ def _check(o, lse, o_ref, lse_ref, what=""):
     lse_err = float((lse - lse_ref).abs().max())
     assert lse_err <= LSE_ATOL, f"{what}: LSE error {lse_err:.3e} > {LSE_ATOL}"
     return float(err.max()), lse_err
+
+
+# attn.variant values: -1 = the library's choice (which depends on head_dim and on how many workgroups the shape gives),
+# 0 = the 128-row kernel, 16 / 32 = the 256-row kernel with eight / four waves (head_dim 128 only)
+KERNELS_D128 = [-1, 0, 16, 32]
+
+
+@pytest.fixture
+def kernel_variant(request):
+    _lib.tune_set("attn.variant", request.param)
+    yield request.param
+    _lib.tune_set("attn.variant", -1)
 
 
 def _run_and_check(B, H, Sq, Sk, D, dtype, causal, seed=0, scale=None):
@@ -78,8 +91,11 @@ def test_throughput_shape_slice_fp16_noncausal():
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 1000), (1, 1, 1000, 64), (3, 5, 191, 191)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
-def test_ragged_and_unequal_lengths(shape, causal, D):
+@pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
+def test_ragged_and_unequal_lengths(shape, causal, D, kernel_variant):
     # sequence lengths that are not multiples of the 128-row / 64-key tiles, Sq != Sk (causal mask is top-left aligned)
+    if D == 64 and kernel_variant > 0:
+        pytest.skip("head_dim 64 has one kernel")
     B, H, Sq, Sk = shape
     _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
 
@@ -87,7 +103,8 @@ def test_ragged_and_unequal_lengths(shape, causal, D):
 @pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
-def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype):
+@pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
+def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype, kernel_variant):
     # head_dim 128 works on 256-row query blocks (two per workgroup when causal) and a four-slot ring of key tiles
     B, H, Sq, Sk = shape
     _run_and_check(B, H, Sq, Sk, 128, dtype, causal, seed=Sq + Sk)
@@ -97,7 +114,10 @@ def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype):
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
-def test_moving_row_maximum(pattern, causal, D, dtype):
+@pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
+def test_moving_row_maximum(pattern, causal, D, dtype, kernel_variant):
+    if D == 64 and kernel_variant > 0:
+        pytest.skip("head_dim 64 has one kernel")
     # scores whose row maximum keeps moving (or sits far above the rest) exercise the rescaling of the running
     # softmax state: keys scaled so that scaled scores span tens of units
     B, H, Sq, Sk = 1, 2, 384, 640
@@ -126,7 +146,8 @@ def test_golden_fixture():
         _check(o, lse, torch.from_numpy(z[f"o_{tag}"]), torch.from_numpy(z[f"lse_{tag}"]), f"golden {tag}")
 
 
-def test_bshd_surface_and_multi_query():
+@pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
+def test_bshd_surface_and_multi_query(kernel_variant):
     # [batch, seqlen, nheads, headdim] inputs (flash_attention_triton.py:734-737); K/V shared across heads via expand,
     # as tests/test_flash_attention_triton.py:71-73 does
     B, S, H, D = 2, 300, 4, 128
@@ -147,7 +168,8 @@ def test_bshd_surface_and_multi_query():
         flash_attn(qd, kd, vd, dropout_p=0.1)
 
 
-def test_non_contiguous_head_slices():
+@pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
+def test_non_contiguous_head_slices(kernel_variant):
     # Q/K/V as slices of one packed [B, S, 3, H, D] projection output
     B, S, H, D = 1, 256, 2, 64
     g = torch.Generator().manual_seed(6)
