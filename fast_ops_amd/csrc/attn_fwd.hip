@@ -8,20 +8,23 @@
 // operand type before P.V (:237), LSE = natural-log logsumexp of the scaled scores (:241-243,255), causal mask
 // top-left aligned with whole key tiles skipped (:149,174-175).
 //
-// Design for CDNA4
-//   * One workgroup = 4 waves = 128 query rows; each wave owns 32 rows. Two workgroups fit a CU (<= 256 VGPRs, 64 KiB
-//     LDS each) so one's softmax (VALU) overlaps the other's MFMA.
-//   * The scores are computed transposed, S^T = K Q^T (A operand = K tile from LDS, B operand = Q^T held in
-//     registers for the whole kernel). In the 32x32 accumulator layout a lane then owns ONE query column and 16 of
-//     the 32 keys, so the row max / row sum are in-lane reductions plus one exchange between the two half-waves,
-//     and the accumulator registers are, as they stand, the B operand of O^T = V^T P^T. P never touches LDS.
+// Two kernels. Common to both:
+//   * The scores are computed transposed, S^T = K Q^T (A operand = K from LDS, B operand = Q^T held in registers for
+//     the whole kernel). In the 32x32 accumulator layout a lane then owns ONE query column and 16 of the 32 keys, so
+//     the row max / row sum are in-lane reductions plus one exchange between the two half-waves, and the accumulator
+//     registers are, as they stand, the B operand of O^T = V^T P^T. P never touches LDS.
 //   * V^T as an A operand needs 8 keys per lane for one d: read from the row-major V tile with the gfx950
 //     transposing LDS load (ds_read_b64_tr_b16).
-//   * K/V tiles (64 keys) go global -> LDS with the direct-to-LDS loads (16 B per lane, no VGPR staging), double
-//     buffered, one barrier per tile. 16-byte chunks are XOR-swizzled inside a row so that both the K reads
-//     (32 rows x one chunk) and the V reads (4 rows x 4 chunks) are free of bank conflicts.
+//   * K/V tiles (64 keys) go global -> LDS with the direct-to-LDS loads (16 B per lane, no VGPR staging).
 //   * Workgroup order: heads are dealt to the 8 XCDs (workgroup ids round-robin over XCDs), each XCD walks one head
-//     at a time with its heaviest (last) causal query blocks first, so an XCD's L2 holds the K/V it is streaming.
+//     at a time, so an XCD's L2 holds the K/V it is streaming.
+// attn_fwd_kernel (head_dim 64, and head_dim 128 for small or very long inputs): one workgroup = 4 waves = 128 query
+//   rows, two workgroups per CU, compiler-scheduled MFMA builtins, tiles double buffered with one barrier per tile,
+//   16-byte chunks XOR-swizzled inside a row so that both the K reads (32 rows x one chunk) and the V reads (4 rows x
+//   4 chunks) are free of bank conflicts; heaviest (last) causal query blocks first.
+// attn_fwd_wide_kernel (head_dim 128): 256 query rows per workgroup, one workgroup per CU, MFMAs as inline assembly
+//   with the accumulators of O and the fragments of Q in AGPRs, a three-deep software pipeline over 32-key sub-tiles
+//   laid out as micro-groups of one MFMA plus its share of everything else; described where it is defined.
 #include <type_traits>
 
 #include "common.hpp"
@@ -626,6 +629,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       for (int r = 0; r < 16; ++r) oacc[i][qb][r] = 0.0f;
   f32x16 S[2][QB];             // scores: sub-tile s, query block qb live in S[s & 1][qb]
   i32x4 PF[2][QB][2];          // P of sub-tile s: PF[s & 1][qb][16-key step]
+  constexpr bool SPREAD_DMA = (DBG & 8) != 0;   // issue the copies of a tile between the MFMAs of its steps instead of at its top
   constexpr int RD = QB == 2 ? 4 : 2;       // must divide the number of fragments of a sub-tile
   static_assert(KSTEPS % RD == 0, "fragment ring");
   i32x4 KF[RD], VF[RD];        // LDS fragment rings, refilled RD fragments ahead of use
@@ -662,7 +666,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // m = -inf); only then (rarely) the step's P is recomputed from the still intact scores against the true maximum,
   // and O and l are rescaled. The result is that of the exact recurrence (flash_attention_triton.py:200-213,241-243)
   // up to rounding.
-  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop) {
+  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop, int dma_tile) {
     // inside the loops the MFMAs go without wait states in front unless the build asked for them (see above)
     typedef AsmMfma<T, !(decltype(in_loop)::value && !FO_MFMA_NOPS)> Mfma;
     constexpr int P = decltype(parity)::value;
@@ -674,7 +678,8 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     // the previous step. Then the mask (if any), then the exponentials.
     constexpr int GMASK = 1;
     constexpr int GE0 = MASK ? 2 : 1;                                   // first group that may read the scores
-    constexpr int NE = G - 2 - GE0;                                     // groups GE0+1 .. G-2 carry the exponentials
+    constexpr int DA = 1;                                               // groups between an exponential and its use
+    constexpr int NE = G - 1 - DA - GE0;                                // groups GE0+1 .. G-1-DA carry the exponentials
     static_assert(NE >= 2, "too few micro-groups");
     // (an opaque copy of the sub-tile index: the variants of this step are selected by branches, and identical address
     // arithmetic in two branches would otherwise be hoisted above them, out of its micro-group)
@@ -707,6 +712,19 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       if constexpr (!HAS_PV) {
         if (g < RD) VF[g] = v_frag(vb1, g);   // first step: the next one expects the first V^T fragments of sub-tile s
       }
+      // -- this group's share of the tile copies (steps of even sub-tiles carry K, of odd ones V)
+      if constexpr (SPREAD_DMA && HAS_QK && HAS_PV) {
+        constexpr int SPACING = (G - 2) / DMA_PER_WAVE;
+        if (g >= 2 && (g - 2) % SPACING == 0 && (g - 2) / SPACING < DMA_PER_WAVE) {
+          const int i = (g - 2) / SPACING;
+          if (dma_tile >= 0) {
+            if (P == 0) dma16_uniform_base(k_src0[i], k_off + (uint32_t)dma_tile * k_tile_bytes,
+                                           smem + (dma_tile & (kRing - 1)) * TILE_BYTES + (wave_s * DMA_PER_WAVE + i) * 1024);
+            else dma16_uniform_base(v_src0[i], v_off + (uint32_t)dma_tile * v_tile_bytes,
+                                    smem + (kRing + (dma_tile & (kRing - 1))) * TILE_BYTES + (wave_s * DMA_PER_WAVE + i) * 1024);
+          }
+        }
+      }
       // -- this group's share of the softmax arithmetic
       if (MASK && g == GMASK) {
         // register r holds key key_base + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); dead iff key > q or key >= Sk,
@@ -735,7 +753,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
           if (!(DBG & 2)) ex[e] = __builtin_amdgcn_exp2f(ex[e]);
           asm volatile("" : "+v"(ex[e]));
         }
-        if (ge + 1 == g) {
+        if (ge + DA == g) {
           psum[b2] += ex[e];                                           // summed in fp32 before rounding (flash_attention_triton.py:203)
           asm volatile("" : "+v"(psum[b2]));
           if (e & 1) {
@@ -795,7 +813,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // ---- tile loop. Tile j runs the steps of sub-tiles 2j and 2j+1; they read K(j), K(j+1), V(j-1), V(j).
   // At its top, copy batches up to (j-2) must have landed - K(j+1) and V(j) are among them - while batch (j-1) may still
   // be in flight; after the barrier every wave is done with tile j-1, so batch j may overwrite K(j-1) and V(j-2).
-  auto tile_top = [&](int j) {
+  auto tile_top = [&](int j) -> bool {
     if (!(DBG & 32)) {
       if (__builtin_expect(last_batch == 2 * DMA_PER_WAVE, 1)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
       else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
@@ -806,7 +824,9 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     // overwrites, and copies are made visible by the vmcnt wait above (it covers this wave's own pieces; the barrier
     // extends that to everyone's).
     if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
+    if (SPREAD_DMA && j + 3 < n_full) { last_batch = 2 * DMA_PER_WAVE; return true; }   // the steps of this tile issue them
     last_batch = (DBG & 1) ? 0 : issue_batch(j);
+    return false;
   };
   // Tiles that need the mask (causal diagonal, keys past the end) are a suffix of the wave's tiles. The hot loops are
   // kept free of alternatives: unmasked tiles, then masked tiles, then the last tile, whose second step has no scores
@@ -816,7 +836,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   if (Sk % kBN != 0) j_mask = min(j_mask, n_tiles - 1);
 
   // first tile: fill the pipeline - S(0) on its own, then a step that has nothing to multiply yet
-  tile_top(0);
+  if (tile_top(0)) { issue(std::false_type{}, 3); issue(std::true_type{}, 2); }
   {
     const uint32_t kb0 = k_lane + sub_base(0), kb1 = k_lane + sub_base(1);
 #pragma unroll
@@ -833,27 +853,28 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     }
   }
   mfma_result_fence_v(S[0]);
-  step(0, P0{}, Y{}, N{}, Y{}, N{});
-  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}); else step(1, P1{}, N{}, Y{}, Y{}, N{});
+  step(0, P0{}, Y{}, N{}, Y{}, N{}, -1);
+  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, -1);
   // The steps above may have parked a few registers in scratch memory. Wait here, visibly to the compiler, for any
   // reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0) wait that executes on
   // every iteration and also drains the copies in flight, which it does not see.
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), nothing else
   int j = 1;
   for (; j < min(j_mask, n_w - 1); ++j) {
-    tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, N{}, Y{});
-    step(2 * j + 1, P1{}, Y{}, Y{}, N{}, Y{});
+    const bool sp = tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, N{}, Y{}, sp ? j + 3 : -1);
+    step(2 * j + 1, P1{}, Y{}, Y{}, N{}, Y{}, sp ? j + 2 : -1);
   }
   for (; j < n_w - 1; ++j) {
-    tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, Y{}, Y{});
-    step(2 * j + 1, P1{}, Y{}, Y{}, Y{}, Y{});
+    const bool sp = tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, Y{}, Y{}, sp ? j + 3 : -1);
+    step(2 * j + 1, P1{}, Y{}, Y{}, Y{}, Y{}, sp ? j + 2 : -1);
   }
   if (j < n_w) {
-    tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, Y{}, N{});
-    step(2 * j + 1, P1{}, N{}, Y{}, Y{}, N{});
+    const bool sp = tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, Y{}, N{}, sp ? j + 3 : -1);
+    step(2 * j + 1, P1{}, N{}, Y{}, Y{}, N{}, -1);
+    if (sp) issue(std::true_type{}, j + 2);
     ++j;
   }
   {
@@ -868,7 +889,8 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     }
   }
   // tiles in which this wave has nothing to do (causal): keep feeding the workgroup's rings
-  for (; j < n_tiles; ++j) tile_top(j);
+  for (; j < n_tiles; ++j)
+    if (tile_top(j)) { issue(std::false_type{}, j + 3); issue(std::true_type{}, j + 2); }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: normalise, write O and LSE
@@ -949,14 +971,9 @@ static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
         case 256 + 2: return launch_wide<T, D, false, 1, 2>(p, stream);
         case 256 + 4: return launch_wide<T, D, false, 1, 4>(p, stream);
         case 256 + 7: return launch_wide<T, D, false, 1, 7>(p, stream);
-        case 256 + 32: return launch_wide<T, D, false, 1, 32>(p, stream);
         case 256 + 64: return launch_wide<T, D, false, 1, 64>(p, stream);
-        case 512 + 1: return launch_wide<T, D, false, 2, 1>(p, stream);
-        case 512 + 2: return launch_wide<T, D, false, 2, 2>(p, stream);
-        case 512 + 4: return launch_wide<T, D, false, 2, 4>(p, stream);
-        case 512 + 32: return launch_wide<T, D, false, 2, 32>(p, stream);
-        case 512 + 64: return launch_wide<T, D, false, 2, 64>(p, stream);
         case 512 + 7: return launch_wide<T, D, false, 2, 7>(p, stream);
+        case 512 + 8: return launch_wide<T, D, false, 2, 8>(p, stream);
         default: return FO_ERR_UNSUPPORTED;
       }
     }
