@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfastops_hip.so")
 
 FO_LION_CHUNK = 8192
-FO_DTYPE_F16, FO_DTYPE_BF16 = 0, 1
+FO_DTYPE_F16, FO_DTYPE_BF16, FO_DTYPE_F32 = 0, 1, 2
 
 
 class FoLionConsts(ctypes.Structure):
@@ -37,6 +37,10 @@ SIGNATURES = {
     "fo_lion_update": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.POINTER(FoLionConsts), ctypes.c_void_p]),
     "fo_lion_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.POINTER(FoLionConsts), ctypes.c_void_p]),
     "fo_lion_fill_chunks": (ctypes.c_int64, [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_void_p]),
+    "fo_lion_make_consts_typed": (ctypes.c_int, [ctypes.c_double] * 4 + [ctypes.c_int, ctypes.c_int, ctypes.POINTER(FoLionConsts)]),
+    "fo_lion_fill_chunks_typed": (ctypes.c_int64, [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "fo_lion_step_typed": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.POINTER(FoLionConsts), ctypes.c_void_p]),
+    "fo_lion_update_typed": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.POINTER(FoLionConsts), ctypes.c_void_p]),
 }
 
 _lock = threading.Lock()

@@ -35,6 +35,7 @@ COMMON_FLAGS = [
 SOURCES = {
     "capi.hip": [],
     "lion.hip": ["-ffp-contract=off"],
+    "lion_typed.hip": ["-ffp-contract=off"],
     # attn_fwd.hip lays its inner loop out as fully unrolled micro-groups; the default size limit for "#pragma unroll"
     # would silently leave them rolled, with their register arrays in scratch memory.
     "attn_fwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],

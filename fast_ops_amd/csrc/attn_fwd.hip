@@ -764,7 +764,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
           }
         }
       }
-      __builtin_amdgcn_sched_barrier(0);
+      if (!(DBG & 128) || (g & 1)) __builtin_amdgcn_sched_barrier(0);
     }
     // -- end of step: did some P get large (or infinite, or NaN from a masked score against m = -inf)?
     bool redo = false;
@@ -972,6 +972,8 @@ static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
         case 256 + 4: return launch_wide<T, D, false, 1, 4>(p, stream);
         case 256 + 7: return launch_wide<T, D, false, 1, 7>(p, stream);
         case 256 + 64: return launch_wide<T, D, false, 1, 64>(p, stream);
+        case 256 + 128: return launch_wide<T, D, false, 1, 128>(p, stream);
+        case 512 + 128: return launch_wide<T, D, false, 2, 128>(p, stream);
         case 512 + 7: return launch_wide<T, D, false, 2, 7>(p, stream);
         case 512 + 8: return launch_wide<T, D, false, 2, 8>(p, stream);
         default: return FO_ERR_UNSUPPORTED;

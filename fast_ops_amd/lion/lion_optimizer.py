@@ -2,15 +2,17 @@
 
 Same constructor, validation, state key and ``step()`` semantics as the reference class
 (fast_ops/lion/lion_optimizer.py:29-76); the arithmetic is that of the reference formula
-(fast_ops/lion/lion_optimizer_ref.py:51,64,65,67) for fp32 parameters and gradients with a bf16 momentum.
+(fast_ops/lion/lion_optimizer_ref.py:51,64,65,67) under PyTorch's type promotion, for parameters/gradients and
+momenta in fp32, fp16 or bf16 (fp32 parameters with a bf16 momentum is the tuned path).
 
 What differs from the reference, on purpose:
 
 * one kernel launch per parameter group instead of one per parameter (lion_optimizer.py:64-76 launches per tensor):
   the tensors of a group are cut into 8192-element chunks whose descriptors live in a device table that is rebuilt
   only when a parameter, gradient or momentum pointer changes;
-* parameters and gradients are fp32 and the momentum is bf16 (the reference kernel requires one half dtype for all
-  three, lion_update.cu:132-135); the momentum dtype for freshly created state is ``exp_avg_dtype``;
+* the reference kernel requires one half dtype for all three tensors (lion_update.cu:132-135); here parameter and
+  momentum dtypes are independent. Freshly created momentum is bf16 for fp32 parameters (the paper's choice) and
+  ``zeros_like(param)`` for half parameters (lion_optimizer.py:68-73) unless ``exp_avg_dtype`` says otherwise;
 * the six scalar constants are computed here in Python double precision and rounded once to fp32, which is what the
   reference formula's Python expressions do.
 """
@@ -46,15 +48,21 @@ def _dense_same_layout(a: Tensor, *others: Tensor) -> bool:
     return True
 
 
-def make_consts(lr: float, betas: Tuple[float, float], weight_decay: float) -> "_lib.FoLionConsts":
+_DTYPE_CODE = {torch.float32: _lib.FO_DTYPE_F32, torch.float16: _lib.FO_DTYPE_F16, torch.bfloat16: _lib.FO_DTYPE_BF16}
+
+
+def make_consts(lr: float, betas: Tuple[float, float], weight_decay: float,
+                p_dtype: torch.dtype = torch.float32, m_dtype: torch.dtype = torch.bfloat16) -> "_lib.FoLionConsts":
     c = _lib.FoLionConsts()
-    _lib.check(_lib.load().fo_lion_make_consts(float(lr), float(betas[0]), float(betas[1]), float(weight_decay), ctypes.byref(c)),
-               "fo_lion_make_consts")
+    _lib.check(_lib.load().fo_lion_make_consts_typed(float(lr), float(betas[0]), float(betas[1]), float(weight_decay),
+                                                     _DTYPE_CODE[p_dtype], _DTYPE_CODE[m_dtype], ctypes.byref(c)),
+               "fo_lion_make_consts_typed")
     return c
 
 
-def build_chunk_table(ptrs: List[Tuple[int, int, int, int]]) -> np.ndarray:
-    """(p_ptr, g_ptr, m_ptr, numel) per tensor -> structured array of fo_lion_chunk descriptors."""
+def build_chunk_table(ptrs: List[Tuple[int, int, int, int]], p_size: int = 4, m_size: int = 2) -> np.ndarray:
+    """(p_ptr, g_ptr, m_ptr, numel) per tensor -> structured array of fo_lion_chunk descriptors; p_size / m_size are
+    the element sizes of parameters (and gradients) and of the momentum."""
     C = _lib.FO_LION_CHUNK
     parts = []
     for p_ptr, g_ptr, m_ptr, numel in ptrs:
@@ -63,9 +71,9 @@ def build_chunk_table(ptrs: List[Tuple[int, int, int, int]]) -> np.ndarray:
         n = (numel + C - 1) // C
         off = np.arange(n, dtype=np.uint64) * np.uint64(C)
         t = np.zeros(n, dtype=_CHUNK_DTYPE)
-        t["p"] = np.uint64(p_ptr) + off * np.uint64(4)
-        t["g"] = np.uint64(g_ptr) + off * np.uint64(4)
-        t["m"] = np.uint64(m_ptr) + off * np.uint64(2)
+        t["p"] = np.uint64(p_ptr) + off * np.uint64(p_size)
+        t["g"] = np.uint64(g_ptr) + off * np.uint64(p_size)
+        t["m"] = np.uint64(m_ptr) + off * np.uint64(m_size)
         t["n"] = np.minimum(np.uint64(C), np.uint64(numel) - off).astype(np.int32)
         parts.append(t)
     return np.concatenate(parts) if parts else np.zeros(0, dtype=_CHUNK_DTYPE)
@@ -74,12 +82,13 @@ def build_chunk_table(ptrs: List[Tuple[int, int, int, int]]) -> np.ndarray:
 def lion_update(param: Tensor, grad: Tensor, exp_avg: Tensor, lr: float, beta1: float, beta2: float, weight_decay: float) -> None:
     """Single-tensor in-place update: the call the reference extension exposes (fast_ops/lion/lion.cpp:4-15)."""
     _check_tensors(param, grad, exp_avg)
-    c = make_consts(lr, (beta1, beta2), weight_decay)
+    c = make_consts(lr, (beta1, beta2), weight_decay, param.dtype, exp_avg.dtype)
     with torch.cuda.device(param.device):
         stream = torch.cuda.current_stream(param.device).cuda_stream
         _lib.check(
-            _lib.load().fo_lion_update(param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), param.numel(), ctypes.byref(c), stream),
-            "fo_lion_update",
+            _lib.load().fo_lion_update_typed(param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), param.numel(),
+                                             _DTYPE_CODE[param.dtype], _DTYPE_CODE[exp_avg.dtype], ctypes.byref(c), stream),
+            "fo_lion_update_typed",
         )
 
 
@@ -88,10 +97,10 @@ def _check_tensors(param: Tensor, grad: Tensor, exp_avg: Tensor) -> None:
         raise RuntimeError("fused Lion runs on the GPU only: parameters, gradients and momentum must be device tensors")
     if not (param.device == grad.device == exp_avg.device):
         raise RuntimeError("parameter, gradient and momentum must live on the same device")
-    if param.dtype != torch.float32 or grad.dtype != torch.float32 or exp_avg.dtype != torch.bfloat16:
+    if param.dtype not in _DTYPE_CODE or exp_avg.dtype not in _DTYPE_CODE or grad.dtype != param.dtype:
         raise RuntimeError(
-            f"unsupported dtypes (param {param.dtype}, grad {grad.dtype}, exp_avg {exp_avg.dtype}): "
-            "this kernel takes float32 parameters and gradients with a bfloat16 momentum"
+            f"unsupported dtypes (param {param.dtype}, grad {grad.dtype}, exp_avg {exp_avg.dtype}): parameters and momentum "
+            "may each be float32, float16 or bfloat16, and the gradient has the parameter's dtype (lion_update.cu:132)"
         )
     if grad.is_sparse:
         raise RuntimeError("Lion does not support sparse gradients")
@@ -109,7 +118,7 @@ class Lion(Optimizer):
         betas: Tuple[float, float] = (0.9, 0.99),
         weight_decay: float = 0.0,
         *,
-        exp_avg_dtype: torch.dtype = torch.bfloat16,
+        exp_avg_dtype: Optional[torch.dtype] = None,
     ) -> None:
         """
         :param params: iterable of parameters to optimize or dicts defining parameter groups
@@ -117,20 +126,20 @@ class Lion(Optimizer):
         :param betas: coefficients of the update interpolation and of the momentum decay
         :param weight_decay: decoupled weight decay coefficient
         :param exp_avg_dtype: dtype of momentum buffers this optimizer creates (state loaded or seeded by the caller
-          keeps its own dtype)
+          keeps its own dtype). None: bfloat16 for float32 parameters, the parameter's dtype otherwise
         """
         # same checks, exception type and messages as lion_optimizer.py:49-52
         if lr <= 0:
             raise RuntimeError(f"expected positive LR, got {lr}")
         if not all(0 <= beta <= 1 for beta in betas):
             raise RuntimeError(f"betas must be between 0 and 1. got {betas}")
-        if exp_avg_dtype != torch.bfloat16:
-            raise RuntimeError(f"exp_avg_dtype {exp_avg_dtype} is not implemented: the fused kernel keeps a bfloat16 momentum")
+        if exp_avg_dtype is not None and exp_avg_dtype not in _DTYPE_CODE:
+            raise RuntimeError(f"exp_avg_dtype {exp_avg_dtype} is not implemented: float32, float16 or bfloat16")
         defaults = {"lr": lr, "betas": betas, "weight_decay": weight_decay}
         super().__init__(params, defaults)
         self._exp_avg_dtype = exp_avg_dtype
-        # (group index, device) -> (key of data pointers, device table tensor, number of chunks)
-        self._tables: Dict[Tuple[int, torch.device], Tuple[tuple, Tensor, int]] = {}
+        # (group index, device, parameter dtype, momentum dtype) -> (key of data pointers, device table tensor, number of chunks)
+        self._tables: Dict[tuple, Tuple[tuple, Tensor, int]] = {}
         _lib.load()   # fail at construction, not at the first step, when the library is missing
 
     @torch.no_grad()
@@ -141,30 +150,33 @@ class Lion(Optimizer):
             lr = group["lr"]
             weight_decay = group["weight_decay"]
             beta1, beta2 = group["betas"]
-            per_device: Dict[torch.device, List[Tuple[int, int, int, int]]] = {}
+            # one launch per (device, parameter dtype, momentum dtype)
+            buckets: Dict[Tuple[torch.device, torch.dtype, torch.dtype], List[Tuple[int, int, int, int]]] = {}
             for param in group["params"]:
                 grad: Optional[Tensor] = param.grad
                 if grad is None:
                     continue
                 state = self.state[param]
                 if "exp_avg" not in state:
-                    # exponential moving average of the gradient (lion_optimizer.py:68-73), kept in bf16
-                    state["exp_avg"] = torch.zeros_like(param, dtype=self._exp_avg_dtype, memory_format=torch.preserve_format)
+                    # exponential moving average of the gradient (lion_optimizer.py:68-73)
+                    dt = self._exp_avg_dtype or (torch.bfloat16 if param.dtype == torch.float32 else param.dtype)
+                    state["exp_avg"] = torch.zeros_like(param, dtype=dt, memory_format=torch.preserve_format)
                 exp_avg: Tensor = state["exp_avg"]
                 _check_tensors(param, grad, exp_avg)
-                per_device.setdefault(param.device, []).append((param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), param.numel()))
-            if not per_device:
-                continue
-            consts = make_consts(lr, (beta1, beta2), weight_decay)
-            for device, ptrs in per_device.items():
+                buckets.setdefault((param.device, param.dtype, exp_avg.dtype), []).append(
+                    (param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), param.numel()))
+            for (device, p_dtype, m_dtype), ptrs in buckets.items():
+                consts = make_consts(lr, (beta1, beta2), weight_decay, p_dtype, m_dtype)
                 key = tuple(ptrs)
-                cached = self._tables.get((gi, device))
+                slot = (gi, device, p_dtype, m_dtype)
+                cached = self._tables.get(slot)
                 if cached is None or cached[0] != key:
-                    table = build_chunk_table(ptrs)
+                    table = build_chunk_table(ptrs, p_dtype.itemsize, m_dtype.itemsize)
                     table_dev = torch.from_numpy(table.view(np.uint8)).to(device)
                     cached = (key, table_dev, int(table.shape[0]))
-                    self._tables[(gi, device)] = cached
+                    self._tables[slot] = cached
                 _, table_dev, n_chunks = cached
                 with torch.cuda.device(device):
                     stream = torch.cuda.current_stream(device).cuda_stream
-                    _lib.check(lib.fo_lion_step(table_dev.data_ptr(), n_chunks, ctypes.byref(consts), stream), "fo_lion_step")
+                    _lib.check(lib.fo_lion_step_typed(table_dev.data_ptr(), n_chunks, _DTYPE_CODE[p_dtype], _DTYPE_CODE[m_dtype],
+                                                      ctypes.byref(consts), stream), "fo_lion_step_typed")

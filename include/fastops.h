@@ -36,7 +36,7 @@ typedef enum fo_status {
   FO_ERR_UNSUPPORTED = -8     /* valid request that this build does not implement */
 } fo_status;
 
-enum { FO_DTYPE_F16 = 0, FO_DTYPE_BF16 = 1 };
+enum { FO_DTYPE_F16 = 0, FO_DTYPE_BF16 = 1, FO_DTYPE_F32 = 2 /* Lion entry points only */ };
 
 /* Human-readable text for a status code; never NULL. */
 const char* fo_strerror(int status);
@@ -122,6 +122,29 @@ int fo_lion_step(const fo_lion_chunk* chunks_dev, int64_t n_chunks, const fo_lio
 /* Host-only helper: fills `out_host[0 .. return value)` with the chunk descriptors of one tensor and returns how many
  * it wrote (ceil(numel / FO_LION_CHUNK)); with out_host == NULL it only counts. */
 int64_t fo_lion_fill_chunks(float* p, const float* g, uint16_t* m, int64_t numel, fo_lion_chunk* out_host);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * Fused Lion step for any parameter/gradient dtype P and momentum dtype M out of FO_DTYPE_F32 / F16 / BF16.
+ * Covers the reference kernel's own case, all three tensors in one half type (lion_update.cu:132-141; exercised by
+ * tests/test_lion_optimizer.py:11-13), and momenta kept in fp32 or fp16. The arithmetic is the reference formula's
+ * (lion_optimizer_ref.py:51,64,65,67) under PyTorch's type promotion: every tensor-valued intermediate is computed
+ * in fp32 and rounded to the dtype the torch expression has (P for p*c and g*(1-beta1), M for m*beta1 and m*beta2,
+ * P if P == M else fp32 for their sum), sign(0) = sign(NaN) = 0, the momentum's add_(grad, alpha) is one fused
+ * multiply-add. P = F32 with M = BF16 is forwarded to fo_lion_update / fo_lion_step.
+ *
+ * fo_lion_make_consts_typed: as fo_lion_make_consts, and when P == M is a half type additionally rounds c_nlr and c_1b2
+ * to that type, as torch does with the `alpha` of an add_ between two tensors of one half type.
+ * fo_lion_fill_chunks_typed / fo_lion_step_typed / fo_lion_update_typed: as their fp32+bf16 counterparts; the pointers
+ * in fo_lion_chunk are then reinterpreted as pointers to P (p, g) and M (m). Alignment: element size; 16-byte aligned
+ * p, g and an m aligned to 16 bytes' worth of elements take the vector path.
+ */
+int fo_lion_make_consts_typed(double lr, double beta1, double beta2, double weight_decay, int p_dtype, int m_dtype,
+                              fo_lion_consts* out_host);
+int64_t fo_lion_fill_chunks_typed(void* p, const void* g, void* m, int64_t numel, int p_dtype, int m_dtype, fo_lion_chunk* out_host);
+int fo_lion_step_typed(const fo_lion_chunk* chunks_dev, int64_t n_chunks, int p_dtype, int m_dtype,
+                       const fo_lion_consts* consts_host, void* stream);
+int fo_lion_update_typed(void* p, const void* g, void* m, int64_t numel, int p_dtype, int m_dtype,
+                         const fo_lion_consts* consts_host, void* stream);
 
 #ifdef __cplusplus
 }

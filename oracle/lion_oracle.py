@@ -24,6 +24,9 @@ The per-element sequence, with the six scalars computed in Python double and rou
     m1 = bf16(f32(f32(m) * c_b2))                       # :67  in-place mul_ rounds to bf16
     m2 = bf16(fma32(c_1b2, g, f32(m1)))                 # :67  add_(grad, alpha=1-beta2) is a fused multiply-add
 
+``lion_step_torch`` takes any dtypes; for the other eight (parameter, momentum) dtype combinations the rounding
+points are spelled out in ``lion_step_explicit_typed``.
+
 Pinned by tests/test_oracle_lion.py: the three restatements agree bit-for-bit on random and adversarial inputs,
 each statement is compared against the single torch op it restates, and the closed-form special cases hold
 (wd = 0, beta1 = 0, beta2 = 0, beta2 = 1, g = m = 0, |delta p| = f32(lr) exactly).
@@ -74,6 +77,41 @@ def lion_step_torch(
         update = exp_avg * beta1 + grad * (1 - beta1)                # :64
         p.add_(torch.sign(update), alpha=-lr)                        # :65
         exp_avg.mul_(beta2).add_(grad, alpha=1 - beta2)              # :67
+
+
+@torch.no_grad()
+def lion_step_explicit_typed(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, lr: float, betas: Tuple[float, float],
+                             weight_decay: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One step for ANY combination of parameter/gradient dtype P and momentum dtype M in {fp32, fp16, bf16}, with
+    every rounding point spelled out: fp32 arithmetic, each tensor-valued intermediate of lion_optimizer_ref.py
+    :51,:64,:65,:67 rounded to the dtype PyTorch's type promotion gives it. Returns (p_new, m_new); inputs untouched.
+
+        p1 = rP(p * c_wd)                         t1 = rM(m * c_b1)      t2 = rP(g * c_1b1)
+        u  = rR(t1 + t2),  R = P if P == M else fp32                     s = sign(u) (0 for 0 and NaN)
+        p2 = rP(p1 + a_nlr * s)                   m2 = rM(fma(a_1b2, g, rM(m * c_b2)))
+
+    a_nlr, a_1b2 are -lr and 1 - beta2 in fp32, except when P == M is a half type: torch converts the ``alpha`` of an
+    add_ between two tensors of one half dtype to that dtype first. The fused multiply-add is emulated in float64
+    (the product of two fp32 values is exact there; a double rounding of the sum is possible in principle).
+    Pinned by tests/test_oracle_lion.py against lion_step_torch (the literal torch statements) for all nine (P, M)."""
+    P, M = p.dtype, m.dtype
+    assert g.dtype == P
+    c_wd, c_b1, c_1b1, c_nlr, c_b2, c_1b2 = (torch.tensor(float(c), dtype=torch.float32) for c in lion_consts(lr, betas, weight_decay))
+    R = P if P == M else torch.float32
+    if P == M and P != torch.float32:
+        c_nlr = c_nlr.to(P).float()
+        c_1b2 = c_1b2.to(P).float()
+    r = lambda x, dt: x.to(dt).float()
+    pf, gf, mf = p.float(), g.float(), m.float()
+    p1 = r(pf * c_wd, P)
+    t1 = r(mf * c_b1, M)
+    t2 = r(gf * c_1b1, P)
+    u = r(t1 + t2, R)
+    s = torch.sign(u)
+    p2 = (p1 + c_nlr * s).to(P)
+    m1 = r(mf * c_b2, M)
+    m2 = (c_1b2.double() * gf.double() + m1.double()).float().to(M)
+    return p2, m2
 
 
 # ---------------------------------------------------------------------------------------------------------------

@@ -217,11 +217,16 @@ def test_param_groups_use_their_own_hyperparameters():
 
 
 def test_wrong_dtypes_and_layouts_raise():
-    a = torch.nn.Parameter(torch.randn(64, device=DEV, dtype=torch.float16))
+    a = torch.nn.Parameter(torch.randn(64, device=DEV, dtype=torch.float64))
     opt = Lion([a])
     a.grad = torch.randn_like(a)
     with pytest.raises(RuntimeError, match="unsupported dtypes"):
         opt.step()
+    b = torch.nn.Parameter(torch.randn(64, device=DEV, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="unsupported dtypes"):   # gradient dtype must be the parameter's (lion_update.cu:132)
+        lion_update(b.detach(), torch.randn(64, device=DEV), torch.zeros(64, device=DEV, dtype=torch.float16), 1e-4, 0.9, 0.99, 0.0)
+    with pytest.raises(RuntimeError, match="exp_avg_dtype"):
+        Lion([b], exp_avg_dtype=torch.float64)
     p = torch.randn(8, 8, device=DEV)
     with pytest.raises(RuntimeError, match="expected tensor to be contiguous"):
         lion_update(p, torch.randn(8, 8, device=DEV).t(), torch.zeros(8, 8, device=DEV, dtype=torch.bfloat16), 1e-4, 0.9, 0.99, 0.0)
@@ -258,3 +263,130 @@ def test_full_size_properties_1p3b():
         assert np.array_equal(_bits32(prm.detach().reshape(-1)[sample]), pc.view(np.uint32))
         assert np.array_equal(_bits16(opt.state[prm]["exp_avg"].reshape(-1)[sample]), mc)
     assert sum(p.numel() for p in params) == 1_308_622_848 and n_each * 78 == 1_308_622_848
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# every (parameter, momentum) dtype combination; fp32 + bf16 above is the tuned path, the other eight share one
+# generic kernel. Oracle: lion_step_explicit_typed (pinned on the CPU against the literal torch statements).
+# ---------------------------------------------------------------------------------------------------------------
+_DTS = [torch.float32, torch.float16, torch.bfloat16]
+
+
+def _same_bits(a, b):
+    a, b = a.detach().cpu(), b.detach().cpu()
+    view = torch.int32 if a.dtype == torch.float32 else torch.int16
+    nan = a.isnan() & b.isnan()        # a NaN stays a NaN; its payload bits are unspecified
+    return bool(torch.equal(a.view(view)[~nan], b.view(view)[~nan]) and torch.equal(a.isnan(), b.isnan()))
+
+
+def _typed_inputs(n, p_dtype, m_dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    p = (torch.randn(n, generator=g) * 0.02).to(p_dtype)
+    m = (torch.randn(n, generator=g) * 1e-3).to(m_dtype)
+    gr = (torch.randn(n, generator=g) * 1e-2).to(p_dtype)
+    return p, gr, m
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 511, 512, 8191, 8192, 8193, 5 * 8192 + 77, (1 << 18) + 5])
+@pytest.mark.parametrize("m_dtype", _DTS, ids=str)
+@pytest.mark.parametrize("p_dtype", _DTS, ids=str)
+def test_typed_single_tensor_bit_exact(p_dtype, m_dtype, n):
+    p, gr, m = _typed_inputs(n, p_dtype, m_dtype, seed=n)
+    if n >= 8:
+        p[:8] = torch.tensor([0.0, -0.0, 1.0, -1.0, 60000.0, 6e-8, 1e-30, float("nan")]).to(p_dtype)
+        m[:3] = 0.0
+        gr[:3] = 0.0                               # u == 0 exactly: sign 0, the parameter only decays
+    pe, me = lo.lion_step_explicit_typed(p, gr, m, **HP)
+    pd, gd, md = p.to(DEV), gr.to(DEV), m.to(DEV)
+    lion_update(pd, gd, md, HP["lr"], *HP["betas"], HP["weight_decay"])
+    torch.cuda.synchronize()
+    assert _same_bits(pd, pe), "parameters differ from the oracle"
+    assert _same_bits(md, me), "momentum differs from the oracle"
+    assert _same_bits(gd, gr), "gradient must not be written"
+
+
+@pytest.mark.parametrize("weight_decay", [0.0, 0.5])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_reference_test_matrix_all_half(weight_decay, dtype):
+    # tests/test_lion_optimizer.py:11-53 at a reduced size (3 x 1024 x 1024 instead of 3 x 8192 x 8192): all tensors in
+    # one half dtype, lr 1e-3, betas (0.9, 0.99), five steps, momentum created by the optimizer as zeros_like(param);
+    # compared after every step with the reference's allclose tolerances against the torch statements AND bit for bit
+    # against the explicit formula
+    hp = dict(lr=1e-3, betas=(0.9, 0.99), weight_decay=weight_decay)
+    g = torch.Generator().manual_seed(0)
+    masters = [torch.randn(1024 * 1024, generator=g).to(dtype) for _ in range(3)]
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in masters]
+    ref_p = [t.clone() for t in masters]
+    ref_m = [torch.zeros_like(t) for t in masters]
+    exp_p = [t.clone() for t in masters]
+    exp_m = [torch.zeros_like(t) for t in masters]
+    opt = Lion(params, **hp)
+    for it in range(5):
+        grads = [torch.randn(1024 * 1024, generator=g).to(dtype) for _ in range(3)]
+        for prm, gr in zip(params, grads):
+            prm.grad = gr.to(DEV)
+        opt.step()
+        lo.lion_step_torch(ref_p, grads, ref_m, **hp)
+        torch.cuda.synchronize()
+        for i in range(3):
+            exp_p[i], exp_m[i] = lo.lion_step_explicit_typed(exp_p[i], grads[i], exp_m[i], **hp)
+            st = opt.state[params[i]]["exp_avg"]
+            assert st.dtype == dtype                      # zeros_like(param), lion_optimizer.py:68-73
+            assert torch.allclose(params[i].detach().cpu(), ref_p[i], rtol=1e-5, atol=1e-2), f"param {i}, iter {it}"
+            assert torch.allclose(st.cpu(), ref_m[i], rtol=1e-5, atol=1e-2), f"exp_avg {i}, iter {it}"
+            assert _same_bits(params[i], exp_p[i]) and _same_bits(st, exp_m[i]), f"bits differ: tensor {i}, iter {it}"
+
+
+def test_typed_mixed_dtypes_in_one_optimizer_and_state_dict():
+    # one parameter group holding fp32, fp16 and bf16 parameters: one launch per (parameter, momentum) dtype pair;
+    # exp_avg_dtype overrides the momentum dtype of new state; state_dict round trip keeps key, dtype and values
+    shapes = [(300, 70), (8192,), (5, 4099)]
+    dts = [torch.float32, torch.float16, torch.bfloat16]
+    g = torch.Generator().manual_seed(3)
+    host_p = [(torch.randn(s, generator=g) * 0.05).to(dt) for s, dt in zip(shapes, dts)]
+    params = [torch.nn.Parameter(t.clone().to(DEV)) for t in host_p]
+    opt = Lion(params, lr=3e-4, betas=(0.95, 0.98), weight_decay=0.01, exp_avg_dtype=torch.float32)
+    exp_p = [t.clone().flatten() for t in host_p]
+    exp_m = [torch.zeros(t.numel(), dtype=torch.float32) for t in host_p]
+    for it in range(3):
+        grads = [(torch.randn(s, generator=g) * 0.01).to(dt) for s, dt in zip(shapes, dts)]
+        for prm, gr in zip(params, grads):
+            prm.grad = gr.to(DEV)
+        opt.step()
+        for i in range(3):
+            exp_p[i], exp_m[i] = lo.lion_step_explicit_typed(exp_p[i], grads[i].flatten(), exp_m[i], 3e-4, (0.95, 0.98), 0.01)
+    torch.cuda.synchronize()
+    for i in range(3):
+        st = opt.state[params[i]]["exp_avg"]
+        assert st.dtype == torch.float32 and st.shape == params[i].shape
+        assert _same_bits(params[i].detach().flatten(), exp_p[i]) and _same_bits(st.flatten(), exp_m[i])
+    sd = opt.state_dict()
+    assert all("exp_avg" in s for s in sd["state"].values())
+    # torch.optim.Optimizer.load_state_dict casts floating-point state to the parameter's dtype (the reference class
+    # inherits the same behaviour); whatever dtype results, the next step must run and agree with the formula
+    opt2 = Lion(params, lr=3e-4, betas=(0.95, 0.98), weight_decay=0.01)
+    opt2.load_state_dict(sd)
+    grads = [(torch.randn(s, generator=g) * 0.01).to(dt) for s, dt in zip(shapes, dts)]
+    for i, prm in enumerate(params):
+        st2 = opt2.state[prm]["exp_avg"]
+        assert st2.dtype == prm.dtype and torch.equal(st2.float(), opt.state[prm]["exp_avg"].to(prm.dtype).float())
+        exp_m[i] = st2.detach().cpu().flatten().clone()
+        prm.grad = grads[i].to(DEV)
+    opt2.step()
+    torch.cuda.synchronize()
+    for i, prm in enumerate(params):
+        pe, me = lo.lion_step_explicit_typed(exp_p[i], grads[i].flatten(), exp_m[i], 3e-4, (0.95, 0.98), 0.01)
+        assert _same_bits(prm.detach().flatten(), pe) and _same_bits(opt2.state[prm]["exp_avg"].flatten(), me)
+
+
+def test_typed_unaligned_views_and_multi_tensor_equivalence():
+    # views at odd element offsets take the element-wise path; a multi-tensor launch equals per-tensor launches
+    for p_dtype, m_dtype in ((torch.float16, torch.float16), (torch.bfloat16, torch.float32), (torch.float32, torch.float32)):
+        n = 20000
+        p, gr, m = _typed_inputs(n + 3, p_dtype, m_dtype, seed=9)
+        pe, me = lo.lion_step_explicit_typed(p[3:], gr[3:], m[1:n + 1], **HP)
+        pd, gd, md = p.to(DEV), gr.to(DEV), m.to(DEV)
+        lion_update(pd[3:], gd[3:], md[1:n + 1], HP["lr"], *HP["betas"], HP["weight_decay"])
+        torch.cuda.synchronize()
+        assert _same_bits(pd[3:], pe) and _same_bits(md[1:n + 1], me)
+        assert _same_bits(pd[:3], p[:3]) and _same_bits(md[:1], m[:1]) and _same_bits(md[n + 1:], m[n + 1:])

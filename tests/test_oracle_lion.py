@@ -182,3 +182,34 @@ def test_golden_fixture():
     for step in range(int(z["steps"])):
         lo.lion_step_c(pc, z["g"][step].copy(), mc, **hp)
     assert _same_bits_f32(pc, z["p_out"]) and np.array_equal(mc, z["m_bits_out"])
+
+
+_DTS = [torch.float32, torch.float16, torch.bfloat16]
+
+
+@pytest.mark.parametrize("m_dtype", _DTS, ids=str)
+@pytest.mark.parametrize("p_dtype", _DTS, ids=str)
+@pytest.mark.parametrize("hp", [dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1), dict(lr=1e-3, betas=(0.95, 0.98), weight_decay=0.0)],
+                         ids=["north-star", "ref-test"])
+def test_explicit_typed_formula_equals_the_torch_statements(p_dtype, m_dtype, hp):
+    # the spelled-out rounding sequence (what the typed kernel implements) against the literal reference statements
+    # executed by torch on the CPU, for all nine dtype combinations, three steps in a row, bit for bit
+    # (n is a power of two on purpose: for two tensors of one half dtype, torch's CPU add_(other, alpha) runs its
+    # vectorised fp32 path on whole vectors and a scalar path - which rounds alpha * other to the half type first - on
+    # the few leftover elements at the end of each thread's range; the vectorised behaviour is the one restated)
+    g0 = torch.Generator().manual_seed(11)
+    n = 1 << 18
+    p = (torch.randn(n, generator=g0) * 0.02).to(p_dtype)
+    m = (torch.randn(n, generator=g0) * 1e-3).to(m_dtype)
+    # adversarial entries: zeros (sign(0) = 0), values that make u cancel exactly, large and tiny magnitudes
+    p[:8] = torch.tensor([0.0, -0.0, 1.0, -1.0, 65504.0, 6e-8, 1e-30, -3.0]).to(p_dtype)
+    m[:4] = 0.0
+    pe, me = p.clone(), m.clone()
+    for step in range(3):
+        gr = (torch.randn(n, generator=g0) * 1e-2).to(p_dtype)
+        gr[:4] = 0.0
+        gr[8] = 0.0
+        pe, me = lo.lion_step_explicit_typed(pe, gr, me, hp["lr"], hp["betas"], hp["weight_decay"])
+        lo.lion_step_torch([p], [gr], [m], hp["lr"], hp["betas"], hp["weight_decay"])
+        assert torch.equal(pe.view(torch.int16 if p_dtype != torch.float32 else torch.int32), p.view(torch.int16 if p_dtype != torch.float32 else torch.int32)), f"params differ at step {step}"
+        assert torch.equal(me.view(torch.int16 if m_dtype != torch.float32 else torch.int32), m.view(torch.int16 if m_dtype != torch.float32 else torch.int32)), f"momentum differs at step {step}"
