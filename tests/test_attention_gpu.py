@@ -137,6 +137,14 @@ def test_moving_row_maximum(pattern, causal, D, dtype, kernel_variant):
     _check(o, lse, o_ref, lse_ref, f"{pattern} D{D} {dtype} causal={causal}")
 
 
+@pytest.mark.parametrize("D", [8, 16, 24, 32, 40, 72, 96, 104, 120])
+@pytest.mark.parametrize("causal", [False, True])
+def test_every_head_dim_of_the_reference_contract(D, causal):
+    # head_dim any multiple of 8 up to 128 (flash_attention.py:61-66); default scale is 1/sqrt(true head_dim)
+    _run_and_check(2, 3, 150, 210, D, torch.float16, causal, seed=D)
+    _run_and_check(1, 2, 97, 97, D, torch.bfloat16, causal, seed=D + 1, scale=0.3)
+
+
 def test_golden_fixture():
     z = np.load(GOLDEN)
     to16 = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16)
@@ -218,8 +226,8 @@ def test_autograd_function_surface():
 
 
 def test_rejected_inputs_raise():
-    q, k, v = (t.to(DEV) for t in _qkv(1, 1, 16, 16, 72, torch.bfloat16))
-    with pytest.raises(RuntimeError, match="head_dim"):
+    q, k, v = (t.to(DEV) for t in _qkv(1, 1, 16, 16, 20, torch.bfloat16))
+    with pytest.raises(RuntimeError, match="multiple of 8"):
         multi_head_attention(q, k, v)
     q, k, v = (t.to(DEV) for t in _qkv(1, 1, 16, 16, 256, torch.bfloat16))
     with pytest.raises(RuntimeError, match="up to 128"):
