@@ -1,0 +1,411 @@
+// FlashAttention backward for gfx950 (MI355X): dQ, dK, dV from Q, K, V, O, dO and the forward's logsumexp.
+//
+// Replaces the backward the reference leaves unimplemented behind its CUDA forward (fast_ops/flash_attention/
+// flash_attention.py:40-45) with what its Triton backward computes (flash_attention_triton.py:273-315 delta pre-pass,
+// :322-638 kernel, :832-958 host): with P = exp(scale * Q K^T - LSE) (masked entries 0),
+//     delta_i = sum_d dO_id O_id      dV = P^T dO      dP = dO V^T      dS = P * (dP - delta) * scale
+//     dQ = dS K                       dK = dS^T Q
+// fp32 scores and accumulators; P and dS are rounded to the operand type before the second GEMMs, as the reference
+// does (:515,:562-563).
+//
+// Three launches, no atomics, no scratch beyond the caller's [B, H, Sq] fp32 `delta` buffer:
+//   1. attn_bwd_delta_kernel: delta.
+//   2. attn_bwd_dq_kernel: one workgroup per 128 query rows (4 waves x 32), walks the key tiles like the forward
+//      kernel. Scores are computed transposed, S^T = K Q^T and dP^T = V dO^T (A operands = K / V rows from LDS, B
+//      operands = Q^T / dO^T held in registers), so a lane owns one query: LSE and delta are per-lane scalars and
+//      dS^T is, as it stands, the B operand of dQ^T = K^T dS^T (A operand via the transposing LDS read of the K tile).
+//   3. attn_bwd_dkdv_kernel: one workgroup per 128 keys (4 waves x 32), walks the query tiles. Here the scores are
+//      computed untransposed, S = Q K^T and dP = dO V^T (A operands = Q / dO rows from LDS, B operands = K^T / V^T
+//      held in registers), so a lane owns one key and P, dS are the B operands of dV^T = dO^T P and dK^T = Q^T dS
+//      (A operands via the transposing LDS read of the dO and Q tiles); per-row LSE and delta come from LDS.
+// Both recompute the scores (seven GEMMs in total instead of the five of an atomics-based single pass).
+// Tiles of 64 rows go global -> LDS with the direct-to-LDS loads, double buffered, one barrier per tile, 16-byte
+// chunks XOR-swizzled inside a row (no bank conflicts), exactly as in the 128-row forward kernel.
+#include "attn_common.hpp"
+
+namespace fo {
+
+constexpr int kBwdWaves = 4;
+constexpr int kBwdRows = 32 * kBwdWaves;   // rows (queries or keys) owned by a workgroup
+constexpr int kBwdTile = 64;               // rows of a streamed tile
+
+struct AttnBwdParams {
+  const void *q, *k, *v, *o, *d_o;
+  const float* lse;
+  float* delta;
+  void *dq, *dk, *dv;
+  int B, H, Sq, Sk;
+  int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];   // element strides: batch, head, sequence
+  float scale, scale_log2e;
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---------------------------------------------------------------------------------------------------------------------
+// delta[b, h, q] = sum_d dO * O   (flash_attention_triton.py:273-315). Eight lanes per row.
+template <typename T, int D>
+__global__ void __launch_bounds__(256) attn_bwd_delta_kernel(const AttnBwdParams prm) {
+  typedef typename Ops<T>::vec8 vec8;
+  const int64_t row = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);
+  const int j = threadIdx.x & 7;
+  const int64_t n_rows = (int64_t)prm.B * prm.H * prm.Sq;
+  float acc = 0.0f;
+  if (row < n_rows) {
+    const int s = (int)(row % prm.Sq);
+    const int bh = (int)(row / prm.Sq);
+    const int b = bh / prm.H, h = bh % prm.H;
+    const T* op = (const T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)s * prm.os[2];
+    const T* gp = (const T*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + (int64_t)s * prm.dos[2];
+#pragma unroll
+    for (int c = j; c < D / 8; c += 8) {
+      const vec8 ov = *(const vec8*)(op + 8 * c), gv = *(const vec8*)(gp + 8 * c);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc += (float)ov[i] * (float)gv[i];
+    }
+  }
+  acc += __shfl_xor(acc, 1);
+  acc += __shfl_xor(acc, 2);
+  acc += __shfl_xor(acc, 4);
+  if (row < n_rows && j == 0) prm.delta[row] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Copy of a 64-row tile (rows row0 .. row0+63 of a [S, D] matrix with row stride `stride`) into LDS by the whole
+// workgroup: per wave D/32 direct-to-LDS instructions. Each instruction fills 1 KiB of LDS with the 64 lanes' pieces
+// back to back, so the swizzle is applied by choosing which global chunk a lane fetches. Rows past the end re-read
+// the last row (callers mask them).
+template <typename T, int D>
+__device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int row0, int S, FO_LDS char* dst, int wave_s, int lane) {
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CHUNKS = ROW_BYTES / 16;
+  constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;
+  constexpr int DMA_PER_WAVE = kBwdTile * ROW_BYTES / 1024 / kBwdWaves;
+#pragma unroll
+  for (int i = 0; i < DMA_PER_WAVE; ++i) {
+    const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane / CHUNKS;
+    const int col = ((lane % CHUNKS) ^ swz<D>(row)) * 8;
+    const int r = min(row0 + row, S - 1);
+    dma16_lane_ptr(base + (int64_t)r * stride + col, dst + (wave_s * DMA_PER_WAVE + i) * 1024);
+  }
+}
+
+// A operand of a 32x32x16 MFMA from a row-major tile in LDS: lane = row l32 of block `blk`, 8 elements at
+// column 16*ks + 8*hh
+template <typename T, int D>
+__device__ __forceinline__ typename Ops<T>::vec8 row_frag(FO_LDS const char* tile, int blk, int ks, int l32, int hh) {
+  const int row = 32 * blk + l32;
+  return *(FO_LDS const typename Ops<T>::vec8*)(tile + row * (D * 2) + (((2 * ks + hh) ^ swz<D>(row)) * 16));
+}
+// A operand = transpose of a tile block: M = 32 columns (d = 32*db ..), K = 16 rows of the tile in the order the 32x32
+// accumulator layout hands them over as a B operand (rows 16*t + 4*hh + {0..3} and + 8)
+template <typename T, int D>
+__device__ __forceinline__ typename Ops<T>::vec8 col_frag(FO_LDS const char* tile, int t, int db, int lane) {
+  const int hh = lane >> 5, L16 = lane & 15, g16 = (lane >> 4) & 1;
+  const int row0 = 16 * t + 4 * hh + (L16 >> 2), row1 = row0 + 8;
+  const int chunk = 4 * db + 2 * g16 + ((L16 & 3) >> 1);
+  const int sub = (L16 & 1) * 8;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(tile + row0 * (D * 2) + ((chunk ^ swz<D>(row0)) * 16) + sub));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(tile + row1 * (D * 2) + ((chunk ^ swz<D>(row1)) * 16) + sub));
+  return __builtin_bit_cast(typename Ops<T>::vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const AttnBwdParams prm) {
+  typedef typename Ops<T>::vec8 vec8;
+  constexpr int TILE_BYTES = kBwdTile * D * 2;
+  constexpr int KSTEPS = D / 16;
+  constexpr int DBLK = D / 32;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // K0 | K1 | V0 | V1
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+  const int n_bh = prm.B * prm.H;
+  const int n_qblk = (prm.Sq + kBwdRows - 1) / kBwdRows;
+  const int bh = blockIdx.x % n_bh;
+  const int qblk = n_qblk - 1 - blockIdx.x / n_bh;   // heaviest causal blocks first
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int q0 = qblk * kBwdRows, q0w = q0 + wave * 32;
+  const int Sq = prm.Sq, Sk = prm.Sk;
+  const T* kbase = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1];
+  const T* vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
+  const int n_tiles = CAUSAL ? (min(Sk, q0 + kBwdRows) + kBwdTile - 1) / kBwdTile : (Sk + kBwdTile - 1) / kBwdTile;
+
+  auto issue = [&](int tile, int buf) {
+    copy_tile64<T, D>(kbase, prm.ks[2], tile * kBwdTile, Sk, smem + buf * TILE_BYTES, wave_s, lane);
+    copy_tile64<T, D>(vbase, prm.vs[2], tile * kBwdTile, Sk, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+  };
+  issue(0, 0);
+
+  // B operands held for the whole kernel: Q^T and dO^T fragments of this lane's query row; its LSE and delta
+  const int qrow = min(q0w + l32, Sq - 1);
+  vec8 qf[KSTEPS], gf[KSTEPS];
+  {
+    const T* qp = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1] + (int64_t)qrow * prm.qs[2] + 8 * hh;
+    const T* gp = (const T*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + (int64_t)qrow * prm.dos[2] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) { qf[ks] = *(const vec8*)(qp + 16 * ks); gf[ks] = *(const vec8*)(gp + 16 * ks); }
+  }
+  const float lse2 = prm.lse[(int64_t)bh * Sq + qrow] * kLog2e;
+  const float delta = prm.delta[(int64_t)bh * Sq + qrow];
+  // (consumed here so that the compiler waits for these loads before the loop: a vmcnt wait inside the loop would
+  // also wait for the tile copies in flight, which it does not see)
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[ks]), "v"(gf[ks]));
+  asm volatile("" ::"v"(lse2), "v"(delta));
+
+  f32x16 acc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  const float c = prm.scale_log2e, scale = prm.scale;
+
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    const int buf = tile & 1;
+    const int key0 = tile * kBwdTile;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tile + 1 < n_tiles) issue(tile + 1, buf ^ 1);
+    if (CAUSAL && key0 > q0w + 31) continue;
+    FO_LDS const char* kt = smem + buf * TILE_BYTES;
+    FO_LDS const char* vt = smem + (2 + buf) * TILE_BYTES;
+
+    f32x16 sacc[2], dpacc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sacc[kb][r] = 0.0f; dpacc[kb][r] = 0.0f; }
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        sacc[kb] = Ops<T>::mfma(row_frag<T, D>(kt, kb, ks, l32, hh), qf[ks], sacc[kb]);      // S^T = K Q^T
+        dpacc[kb] = Ops<T>::mfma(row_frag<T, D>(vt, kb, ks, l32, hh), gf[ks], dpacc[kb]);    // dP^T = V dO^T
+      }
+    // register r of block kb holds key key0 + 32*kb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); dead iff
+    // key > q or key >= Sk
+    vec8 dsf[4];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int key_base = key0 + 32 * kb + 4 * hh;
+      int lim = key_base - Sk + 1;
+      if (CAUSAL) lim = max(lim, key_base - (q0w + l32));
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const bool dead = lim > -((r & 3) + 8 * (r >> 2));
+        const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -lse2));
+        dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dpacc[kb][r] - delta) * scale);
+      }
+    }
+    // dQ^T += K^T dS^T : four 16-key steps x DBLK d-blocks
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int db = 0; db < DBLK; ++db) acc[db] = Ops<T>::mfma(col_frag<T, D>(kt, t, db, lane), dsf[t], acc[db]);
+  }
+
+  const int qi = q0w + l32;
+  if (qi < Sq) {
+    T* op = (T*)prm.dq + b * prm.dqs[0] + h * prm.dqs[1] + (int64_t)qi * prm.dqs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        vec4 o4;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o4[u] = (T)acc[db][rg * 4 + u];
+        *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const AttnBwdParams prm) {
+  typedef typename Ops<T>::vec8 vec8;
+  constexpr int TILE_BYTES = kBwdTile * D * 2;
+  constexpr int KSTEPS = D / 16;
+  constexpr int DBLK = D / 32;
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q0 | Q1 | dO0 | dO1 | lse[2][64] | delta[2][64]
+  FO_LDS float* rowvals = (FO_LDS float*)(smem + 4 * TILE_BYTES);
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+  const int n_bh = prm.B * prm.H;
+  const int bh = blockIdx.x % n_bh;
+  const int kblk = blockIdx.x / n_bh;                 // key block 0 has the most queries when causal: heaviest first
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int k0 = kblk * kBwdRows, k0w = k0 + wave * 32;
+  const int Sq = prm.Sq, Sk = prm.Sk;
+  const T* qbase = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  const T* gbase = (const T*)prm.d_o + b * prm.dos[0] + h * prm.dos[1];
+  const int n_qt = (Sq + kBwdTile - 1) / kBwdTile;
+  const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;   // queries before the block's first key never attend it
+
+  auto issue = [&](int qt, int buf) {
+    copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
+    copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    // per-row LSE and delta of the tile, 4 bytes per lane, also straight into LDS (a load the compiler can see would
+    // make it wait for the tile copies as well); rows past the end re-read the last row and are masked below
+    if (wave_s < 2) {
+      const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
+      dma4_lane_ptr((wave_s == 0 ? prm.lse : (const float*)prm.delta) + at, rowvals + (2 * wave_s + buf) * kBwdTile);
+    }
+  };
+  if (qt0 < n_qt) issue(qt0, 0);
+
+  // B operands held for the whole kernel: K^T and V^T fragments of this lane's key
+  const int key = k0w + l32;
+  const int krow = min(key, Sk - 1);
+  vec8 kf[KSTEPS], vf[KSTEPS];
+  {
+    const T* kp = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1] + (int64_t)krow * prm.ks[2] + 8 * hh;
+    const T* vp = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1] + (int64_t)krow * prm.vs[2] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) { kf[ks] = *(const vec8*)(kp + 16 * ks); vf[ks] = *(const vec8*)(vp + 16 * ks); }
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(kf[ks]), "v"(vf[ks]));
+  }
+
+  f32x16 dkacc[DBLK], dvacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.0f; dvacc[i][r] = 0.0f; }
+  const float c = prm.scale_log2e, scale = prm.scale;
+
+  for (int qt = qt0; qt < n_qt; ++qt) {
+    const int buf = (qt - qt0) & 1;
+    const int q0t = qt * kBwdTile;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (qt + 1 < n_qt) issue(qt + 1, buf ^ 1);
+    FO_LDS const char* qtile = smem + buf * TILE_BYTES;
+    FO_LDS const char* gtile = smem + (2 + buf) * TILE_BYTES;
+    FO_LDS const float* lse_t = rowvals + buf * kBwdTile;
+    FO_LDS const float* del_t = rowvals + (2 + buf) * kBwdTile;
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      if (CAUSAL && q0t + 32 * qb + 31 < k0w) continue;   // every query of the block is before every key of this wave
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sacc[r] = 0.0f; dpacc[r] = 0.0f; }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        sacc = Ops<T>::mfma(row_frag<T, D>(qtile, qb, ks, l32, hh), kf[ks], sacc);      // S = Q K^T
+        dpacc = Ops<T>::mfma(row_frag<T, D>(gtile, qb, ks, l32, hh), vf[ks], dpacc);    // dP = dO V^T
+      }
+      // register r holds query q0t + 32*qb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); dead iff key > query
+      // or the query is past the end
+      const int lim = CAUSAL ? key - (q0t + 32 * qb + 4 * hh) : 0;
+      const int lim_end = Sq - (q0t + 32 * qb + 4 * hh);
+      vec8 pf[2], dsf[2];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 l4 = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * j + 4 * hh);
+        const f32x4 d4 = *(FO_LDS const f32x4*)(del_t + 32 * qb + 8 * j + 4 * hh);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int r = 4 * j + u;
+          const bool dead = (u + 8 * j) < lim || (u + 8 * j) >= lim_end;
+          const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], c, -l4[u] * kLog2e));
+          pf[r >> 3][r & 7] = (T)p;
+          dsf[r >> 3][r & 7] = (T)(p * (dpacc[r] - d4[u]) * scale);
+        }
+      }
+      // dV^T += dO^T P and dK^T += Q^T dS : two 16-query steps x DBLK d-blocks
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db) {
+          dvacc[db] = Ops<T>::mfma(col_frag<T, D>(gtile, 2 * qb + t, db, lane), pf[t], dvacc[db]);
+          dkacc[db] = Ops<T>::mfma(col_frag<T, D>(qtile, 2 * qb + t, db, lane), dsf[t], dkacc[db]);
+        }
+    }
+  }
+
+  if (key < Sk) {
+    T* kp = (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1] + (int64_t)key * prm.dks[2];
+    T* vp = (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1] + (int64_t)key * prm.dvs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        vec4 k4, v4;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { k4[u] = (T)dkacc[db][rg * 4 + u]; v4[u] = (T)dvacc[db][rg * 4 + u]; }
+        *(vec4*)(kp + 32 * db + 8 * rg + 4 * hh) = k4;
+        *(vec4*)(vp + 32 * db + 8 * rg + 4 * hh) = v4;
+      }
+  }
+}
+
+template <typename T, int D, bool CAUSAL>
+static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
+  const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
+  const int64_t n_bh = (int64_t)p.B * p.H;
+  const int64_t g_delta = (n_rows + 31) / 32;
+  const int64_t g_dq = ((p.Sq + kBwdRows - 1) / kBwdRows) * n_bh;
+  const int64_t g_dkdv = ((p.Sk + kBwdRows - 1) / kBwdRows) * n_bh;
+  if (g_delta > 0x7FFFFFFFll || g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
+  const size_t lds_dq = 4 * (size_t)kBwdTile * D * 2;
+  const size_t lds_dkdv = lds_dq + 4 * kBwdTile * sizeof(float);
+  static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
+  static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+  if (a1 != hipSuccess || a2 != hipSuccess) return FO_ERR_LAUNCH;
+  attn_bwd_delta_kernel<T, D><<<(unsigned)g_delta, 256, 0, s>>>(p);
+  attn_bwd_dq_kernel<T, D, CAUSAL><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
+  attn_bwd_dkdv_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
+  return launch_status();
+}
+
+}  // namespace fo
+
+using namespace fo;
+
+extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                           float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                           const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream) {
+  if (!q || !k || !v || !o || !d_o || !lse || !delta_ws || !dq || !dk || !dv || !strides_host) return FO_ERR_NULL_POINTER;
+  for (int t = 0; t < 8; ++t)
+    if (!strides_host[t]) return FO_ERR_NULL_POINTER;
+  if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
+  if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
+  if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || (int64_t)B * H * Sq > (1ll << 40)) return FO_ERR_BAD_SHAPE;
+  for (int t = 0; t < 8; ++t) {
+    // rows start on 16-byte boundaries (8 elements); only the inputs K and V may repeat a head (stride 0 = multi-query)
+    for (int i = 0; i < 3; ++i)
+      if (strides_host[t][i] < 0 || (strides_host[t][i] % 8) != 0) return FO_ERR_BAD_STRIDE;
+    if (strides_host[t][2] < D) return FO_ERR_BAD_STRIDE;
+    const bool output = t >= 5;
+    if (output && ((strides_host[t][0] == 0 && B > 1) || (strides_host[t][1] == 0 && H > 1))) return FO_ERR_BAD_STRIDE;
+  }
+  const uintptr_t all = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv;
+  if (all & 15u) return FO_ERR_MISALIGNED;
+  if (((uintptr_t)lse | (uintptr_t)delta_ws) & 3u) return FO_ERR_MISALIGNED;
+  if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;
+
+  AttnBwdParams p;
+  p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse; p.delta = delta_ws; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  int64_t* dst[8] = {p.qs, p.ks, p.vs, p.os, p.dos, p.dqs, p.dks, p.dvs};
+  for (int t = 0; t < 8; ++t)
+    for (int i = 0; i < 3; ++i) dst[t][i] = strides_host[t][i];
+  p.scale = softmax_scale;
+  p.scale_log2e = softmax_scale * kLog2e;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool c = causal != 0;
+#define FO_BWD(T, DD) (c ? launch_bwd<T, DD, true>(p, s) : launch_bwd<T, DD, false>(p, s))
+  if (dtype == FO_DTYPE_BF16) return D == 128 ? FO_BWD(__bf16, 128) : FO_BWD(__bf16, 64);
+  return D == 128 ? FO_BWD(_Float16, 128) : FO_BWD(_Float16, 64);
+#undef FO_BWD
+}

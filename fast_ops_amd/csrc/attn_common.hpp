@@ -1,0 +1,55 @@
+// Helpers shared by the attention kernels (forward and backward) of libfastops_hip.so.
+#pragma once
+#include "common.hpp"
+
+namespace fo {
+
+#define FO_LDS __attribute__((address_space(3)))
+#define FO_GLOBAL __attribute__((address_space(1)))
+
+template <typename T> struct Ops;
+template <> struct Ops<__bf16> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Ops<_Float16> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+
+// swizzle of 16-byte chunks inside a tile row; `row` is the row inside the tile
+template <int D>
+__device__ __forceinline__ int swz(int row) {
+  if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);              // 16 chunks per 256-byte row
+  else { const int R = row >> 1; return ((R & 1) << 2) | ((R >> 1) & 3); }          // 8 chunks per 128-byte row
+}
+
+__device__ __forceinline__ float half_swap(float x) {
+  // value held by the lane 32 positions away
+  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), false, false);
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
+
+// 16 bytes per lane, global -> LDS without passing through registers. LDS receives the 64 lanes' pieces back to back
+// starting at `dst` (wave-uniform); the global address is per lane.
+// (hipcc also parses device functions in its host pass, where GCN assembly cannot be checked: the bodies exist in the
+// device pass only.)
+__device__ __forceinline__ void dma16_uniform_base(const void* base, uint32_t byte_off, FO_LDS void* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"((uint32_t)(uintptr_t)dst), "v"(byte_off), "s"(base) : "memory", "m0");
+#endif
+}
+__device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"((uint32_t)(uintptr_t)dst), "v"(ptr) : "memory", "m0");
+#endif
+}
+
+// the same with 4 bytes per lane (LDS receives 256 bytes)
+__device__ __forceinline__ void dma4_lane_ptr(const void* ptr, FO_LDS void* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"((uint32_t)(uintptr_t)dst), "v"(ptr) : "memory", "m0");
+#endif
+}
+
+}  // namespace fo

@@ -4,7 +4,9 @@
 [B, H, M, D] queries, [B, H, N, D] keys and values, fp16 or bf16, returns [B, H, M, D]. The reference's CUDA kernel
 behind that call is unfinished and returns zeros (flash_attention_fwd.cu:120-151,158); this one computes
 softmax(scale * Q K^T + mask) V with the numerics of the reference's working Triton forward
-(flash_attention_triton.py:128-255) and can return the logsumexp that forward also produces (:255,771).
+(flash_attention_triton.py:128-255) and can return the logsumexp that forward also produces (:255,771). The backward
+the reference leaves unimplemented (flash_attention.py:40-45) is implemented too, after the Triton backward
+(flash_attention_triton.py:832-958), so ``FlashAttentionFunction`` is trainable.
 
 Keyword-only extras that the reference's README promises or its Triton surface already has
 (flash_attention/README.md:34-38, flash_attention_triton.py:722-731): ``causal``, ``softmax_scale``, ``return_lse``.
@@ -82,6 +84,48 @@ def attn_fwd_strided(
     return o, lse
 
 
+def attn_bwd_strided(
+    q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor, d_o: Tensor, dims: Tuple[int, int, int, int], causal: bool,
+    softmax_scale: Optional[float],
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Launches fo_attn_bwd. Returns (dQ, dK, dV) with the shapes and dtypes of q, k, v (dense; a K/V whose heads are
+    an expanded view gets a full-size gradient, which autograd then reduces)."""
+    _check_inputs(q, k, v)
+    ib, ih, is_, id_ = dims
+    B, H, Sq, D = q.shape[ib], q.shape[ih], q.shape[is_], q.shape[id_]
+    Sk = k.shape[is_]
+    scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(D)
+    if d_o.dtype != q.dtype or d_o.shape != q.shape:
+        raise RuntimeError(f"dO must have the output's shape and dtype, got {tuple(d_o.shape)} {d_o.dtype}")
+    if D not in (64, 128):
+        # same zero padding as the forward; O's padded columns are zero, so delta and the padded gradient columns are too
+        Dp = 64 if D < 64 else 128
+        pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
+        dq, dk, dv = attn_bwd_strided(pad(q), pad(k), pad(v), pad(o), lse, pad(d_o), dims, causal, scale)
+        return tuple(t.narrow(id_, 0, D).contiguous() for t in (dq, dk, dv))
+    if d_o.stride(-1) != 1 or any(s % 8 for s in d_o.stride()[:-1]):
+        d_o = d_o.contiguous()
+    if o.stride(-1) != 1:
+        o = o.contiguous()
+    lse = lse.contiguous()
+    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+    delta = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    tensors = (q, k, v, o, d_o, dq, dk, dv)
+    arrays = [_I64x3(t.stride(ib), t.stride(ih), t.stride(is_)) for t in tensors]
+    ptrs = (ctypes.POINTER(ctypes.c_int64) * 8)(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in arrays])
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        status = _lib.load().fo_attn_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, Sq, Sk, D, ptrs, scale, int(bool(causal)),
+            _DTYPE_CODE[q.dtype], stream,
+        )
+    _lib.check(status, "fo_attn_bwd")
+    return dq, dk, dv
+
+
 class FlashAttentionFunction(Function):
     @staticmethod
     def forward(ctx, Q: Tensor, K: Tensor, V: Tensor, causal: bool = False, softmax_scale: Optional[float] = None,
@@ -102,9 +146,33 @@ class FlashAttentionFunction(Function):
         return o
 
     @staticmethod
-    def backward(ctx, *grads):
-        """:param dO: (B, H, M, D) Output gradient. Not implemented, as in the reference (flash_attention.py:40-45)."""
-        raise NotImplementedError
+    def backward(ctx, dO: Tensor, *unused):
+        """:param dO: (B, H, M, D) Output gradient. The reference leaves this unimplemented (flash_attention.py:40-45);
+        here it is what the reference's Triton backward computes (flash_attention_triton.py:832-958)."""
+        Q, K, V, o, lse = ctx.saved_tensors
+        dq, dk, dv = attn_bwd_strided(Q, K, V, o, lse, dO, (0, 1, 2, 3), ctx.causal, ctx.softmax_scale)
+        return dq, dk, dv, None, None, None
+
+
+class _FlashAttnBSHD(Function):
+    """flash_attn's autograd node: the same kernels on [batch, seqlen, nheads, headdim] tensors."""
+
+    @staticmethod
+    def forward(ctx, q: Tensor, k: Tensor, v: Tensor, causal: bool, softmax_scale: Optional[float], return_lse: bool):
+        o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.causal = causal
+        ctx.softmax_scale = softmax_scale
+        if return_lse:
+            ctx.mark_non_differentiable(lse)
+            return o, lse
+        return o
+
+    @staticmethod
+    def backward(ctx, dO: Tensor, *unused):
+        q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv = attn_bwd_strided(q, k, v, o, lse, dO, (0, 2, 1, 3), ctx.causal, ctx.softmax_scale)
+        return dq, dk, dv, None, None, None
 
 
 def multi_head_attention(
@@ -132,10 +200,9 @@ def flash_attn(
     softmax_scale: Optional[float] = None, return_lse: bool = False,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """The [batch, seqlen, nheads, headdim] surface of flash_attn_triton (flash_attention_triton.py:722-737,961),
-    forward only. Bias and dropout are not implemented and raise."""
+    differentiable. Bias and dropout are not implemented and raise."""
     if bias is not None:
         raise RuntimeError("attention bias is not implemented")
     if dropout_p != 0.0:
         raise RuntimeError("attention dropout is not implemented")
-    o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale)
-    return (o, lse) if return_lse else o
+    return _FlashAttnBSHD.apply(q, k, v, causal, softmax_scale, return_lse)

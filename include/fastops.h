@@ -77,6 +77,27 @@ int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
                 float softmax_scale, int causal, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * FlashAttention backward: dQ, dK, dV.
+ * Implements the backward that flash_attention.py:40-45 leaves unimplemented, with the arithmetic of the reference's
+ * Triton backward (flash_attention_triton.py:273-315 delta pre-pass, :322-638 kernel, :832-958 host): with
+ * P = exp(scale * Q K^T - LSE) (masked entries 0), delta_i = sum_d dO_id O_id,
+ *     dV = P^T dO,   dS = P * (dO V^T - delta) * scale,   dQ = dS K,   dK = dS^T Q;
+ * fp32 scores and accumulators, P and dS rounded to the operand type before the second products.
+ *
+ *   q, k, v, o, lse     as passed to / produced by fo_attn_fwd (lse is required here)
+ *   d_o                 [B, H, Sq, D] gradient of the output
+ *   delta_ws            [B, H, Sq] fp32, contiguous: workspace supplied by the caller, overwritten
+ *   dq / dk, dv         [B, H, Sq, D] / [B, H, Sk, D], written for every element; never read
+ *   strides_host        eight pointers to three element strides each (batch, head, sequence; head_dim stride 1), in
+ *                       the order q, k, v, o, d_o, dq, dk, dv. Only the inputs may repeat a batch or head (stride 0).
+ * Same requirements as fo_attn_fwd (D in {64, 128}, 16-byte aligned pointers and rows, scale finite and > 0).
+ * Three launches on `stream`; no atomics, results are deterministic.
+ */
+int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * Fused Lion step: fp32 parameters, fp32 gradients, bf16 momentum, one pass.
  * Per element, in this order and with these rounding points (lion_optimizer_ref.py:51,64,65,67):
  *     p1 = p * c_wd

@@ -12,6 +12,9 @@ Restates, with torch CPU ops in fp32, what the reference defines:
   ``online_softmax_tiles`` so that tests can show recurrence == closed form, including the running reference
   being ``lse_i`` rather than ``m_i``.
 
+* backward: ``attention_bwd_oracle`` - the closed-form gradients of the same expression
+  (``flash_attention_triton.py:273-315,497-578``).
+
 Layout is the drop-in surface's: Q [B,H,M,D], K/V [B,H,N,D] (``flash_attention.py:30-37``).
 
 Pinned by tests/test_oracle_attention.py against: torch.nn.functional.scaled_dot_product_attention (independent
@@ -61,6 +64,47 @@ def attention_fwd_oracle(
                 attn = torch.softmax(scores, dim=-1)                          # attention_ref.py:59
                 out[b, h, m0:m1] = attn @ vf[b, h]                            # attention_ref.py:67
     return out, lse
+
+
+def attention_bwd_oracle(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    d_o: torch.Tensor,
+    causal: bool = False,
+    softmax_scale: Optional[float] = None,
+    dtype: torch.dtype = torch.float32,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gradients of sum(O * dO) with respect to Q, K, V, in closed form, one (batch, head) at a time:
+
+        P = softmax(scale * Q K^T + mask)        dV = P^T dO           dP = dO V^T
+        delta_i = sum_d dO_id O_id               dS = P * (dP - delta) dQ = scale * dS K        dK = scale * dS^T Q
+
+    which is what the reference's backward computes tile by tile (flash_attention_triton.py:273-315 delta pre-pass,
+    :497-578 per-tile dv / dp / ds / dk / dq) and what autograd gives for attention_ref.py:41-67. ``dtype`` is the
+    arithmetic type (fp32 for the oracle proper, float64 to pin it). Returns (dQ, dK, dV) in ``dtype`` on the CPU.
+    Pinned by tests/test_oracle_attention.py against torch.autograd on the forward expression in float64."""
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    qf, kf, vf, gf = (t.to(dtype).cpu() for t in (q, k, v, d_o))
+    dq, dk, dv = torch.zeros_like(qf), torch.zeros_like(kf), torch.zeros_like(vf)
+    for b in range(B):
+        for h in range(H):
+            s = (qf[b, h] * scale) @ kf[b, h].t()
+            if causal:
+                rows = torch.arange(M).unsqueeze(1)
+                cols = torch.arange(N).unsqueeze(0)
+                s = s.masked_fill(cols > rows, float("-inf"))
+            p = torch.softmax(s, dim=-1)
+            o = p @ vf[b, h]
+            dv[b, h] = p.t() @ gf[b, h]
+            dp = gf[b, h] @ vf[b, h].t()
+            delta = (gf[b, h] * o).sum(dim=-1, keepdim=True)
+            ds = p * (dp - delta)
+            dq[b, h] = (ds @ kf[b, h]) * scale
+            dk[b, h] = (ds.t() @ qf[b, h]) * scale
+    return dq, dk, dv
 
 
 def online_softmax_tiles(

@@ -1,0 +1,136 @@
+"""Parity of the attention backward kernels (through the C ABI and the autograd Function) with the CPU oracle.
+
+Criterion: the reference's own (tests/test_flash_attention_triton.py:137-141) - the error against the fp32 closed form
+must not exceed twice the error of a plain half-precision PyTorch implementation of the same expression, plus an
+absolute floor of 1e-3 of the gradient's magnitude for the cases where that implementation happens to be almost exact.
+Inputs are drawn on the CPU from a seeded generator, rounded to the operand type, then copied."""
+import math
+
+import pytest
+import torch
+
+from fast_ops.flash_attention.flash_attention import FlashAttentionFunction, flash_attn, multi_head_attention
+from oracle.attention_oracle import attention_bwd_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _inputs(B, H, Sq, Sk, D, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    k = torch.randn(B, H, Sk, D, generator=g).to(dtype)
+    v = torch.randn(B, H, Sk, D, generator=g).to(dtype)
+    go = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    return q, k, v, go
+
+
+def _half_precision_torch(q, k, v, go, causal, scale):
+    """The expression evaluated by autograd with tensors of the operand type (matmuls accumulate in fp32 inside, results
+    and the softmax are rounded to the operand type): the 'PyTorch implementation' of the reference's criterion."""
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    s = (qa * scale) @ ka.transpose(-1, -2)
+    if causal:
+        M, N = q.shape[2], k.shape[2]
+        s = s.masked_fill(torch.arange(N)[None, :] > torch.arange(M)[:, None], float("-inf"))
+    o = torch.softmax(s.float(), dim=-1).to(q.dtype) @ va
+    return torch.autograd.grad(o, (qa, ka, va), go)
+
+
+def _check(got, ref, pt, what):
+    for name, a, r, p in zip(("dQ", "dK", "dV"), got, ref, pt):
+        a = a.float().cpu()
+        err = (a - r).abs().max().item()
+        base = (p.float() - r).abs().max().item()
+        bound = 2.0 * base + 1e-3 * max(1.0, r.abs().max().item())
+        assert math.isfinite(err) and err <= bound, f"{what} {name}: error {err:.3e} > 2 x {base:.3e} + floor"
+
+
+def _run(B, H, Sq, Sk, D, dtype, causal, seed=0, scale=None):
+    q, k, v, go = _inputs(B, H, Sq, Sk, D, dtype, seed)
+    sc = scale if scale is not None else 1.0 / math.sqrt(D)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal, softmax_scale=sc)
+    pt = _half_precision_torch(q, k, v, go, causal, sc)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o = multi_head_attention(qd, kd, vd, causal=causal, softmax_scale=scale)
+    got = torch.autograd.grad(o, (qd, kd, vd), go.to(DEV))
+    torch.cuda.synchronize()
+    assert all(gr.dtype == dtype and gr.shape == t.shape for gr, t in zip(got, (q, k, v)))
+    _check(got, ref, pt, f"B{B} H{H} Sq{Sq} Sk{Sk} D{D} {dtype} causal={causal}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_dtype_causal_headdim_grid(dtype, causal, D):
+    _run(2, 3, 256, 256, D, dtype, causal, seed=D)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 300),
+                                   (1, 1, 300, 64), (2, 2, 191, 191), (1, 1, 385, 513)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_ragged_and_unequal_lengths(shape, causal, D):
+    # lengths that are not multiples of the 128-row blocks / 64-row tiles, Sq != Sk (causal mask top-left aligned: keys
+    # beyond the last query get exactly zero gradient)
+    B, H, Sq, Sk = shape
+    _run(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
+
+
+def test_config2_gpt2_small_shape_slice():
+    _run(2, 12, 1024, 1024, 64, torch.bfloat16, True, seed=2)
+
+
+@pytest.mark.parametrize("D", [8, 40, 96])
+def test_other_head_dims_by_padding(D):
+    _run(1, 2, 150, 210, D, torch.float16, True, seed=D)
+    _run(1, 2, 97, 97, D, torch.bfloat16, False, seed=D + 1, scale=0.3)
+
+
+def test_keys_no_query_attends_get_zero_gradient():
+    q, k, v, go = _inputs(1, 2, 100, 400, 128, torch.bfloat16, 5)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o = multi_head_attention(qd, kd, vd, causal=True)
+    _, dk, dv = torch.autograd.grad(o, (qd, kd, vd), go.to(DEV))
+    assert float(dk[:, :, 100:].abs().max()) == 0.0 and float(dv[:, :, 100:].abs().max()) == 0.0
+
+
+def test_bshd_surface_multi_query_and_packed_views():
+    # [batch, seqlen, nheads, headdim] inputs; K/V shared across heads through expand: autograd sums the per-head
+    # gradients the kernel writes; Q/K/V as slices of one packed projection output
+    B, S, H, D = 2, 200, 4, 64
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16)
+    kv = torch.randn(B, S, 2, 1, D, generator=g).to(torch.bfloat16)
+    go = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16)
+    k1, v1 = kv.unbind(2)
+    kx, vx = k1.expand(B, S, H, D), v1.expand(B, S, H, D)
+    tr = lambda t: t.transpose(1, 2)
+    dq_r, dk_r, dv_r = attention_bwd_oracle(tr(q), tr(kx), tr(vx), tr(go), causal=True)
+    pt = _half_precision_torch(tr(q).contiguous(), tr(kx).contiguous(), tr(vx).contiguous(), tr(go).contiguous(), True, 1 / math.sqrt(D))
+    qd = q.to(DEV).requires_grad_(True)
+    kvd = kv.to(DEV).requires_grad_(True)
+    kd, vd = (t.expand(B, S, H, D) for t in kvd.unbind(2))
+    o = flash_attn(qd, kd, vd, causal=True)
+    dq, dkv = torch.autograd.grad(o, (qd, kvd), go.to(DEV))
+    ref = (tr(dq_r), tr(dk_r).sum(2, keepdim=True), tr(dv_r).sum(2, keepdim=True))
+    ptr = (tr(pt[0]), tr(pt[1]).float().sum(2, keepdim=True), tr(pt[2]).float().sum(2, keepdim=True))
+    _check((dq, dkv[:, :, 0], dkv[:, :, 1]), ref, ptr, "BSHD multi-query")
+    # packed projection
+    qkv = torch.randn(B, S, 3, H, D, generator=g).to(torch.bfloat16)
+    qkvd = qkv.to(DEV).requires_grad_(True)
+    o = flash_attn(qkvd[:, :, 0], qkvd[:, :, 1], qkvd[:, :, 2], causal=False)
+    (dqkv,) = torch.autograd.grad(o, (qkvd,), go.to(DEV))
+    r = attention_bwd_oracle(tr(qkv[:, :, 0]), tr(qkv[:, :, 1]), tr(qkv[:, :, 2]), tr(go), causal=False)
+    p = _half_precision_torch(*(tr(qkv[:, :, i]).contiguous() for i in range(3)), tr(go).contiguous(), False, 1 / math.sqrt(D))
+    _check(tuple(dqkv[:, :, i] for i in range(3)), tuple(tr(x) for x in r), tuple(tr(x) for x in p), "packed qkv")
+
+
+def test_gradients_are_deterministic():
+    q, k, v, go = _inputs(2, 4, 512, 512, 128, torch.bfloat16, 9)
+    outs = []
+    for _ in range(2):
+        qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+        o = FlashAttentionFunction.apply(qd, kd, vd, True)
+        outs.append(torch.autograd.grad(o, (qd, kd, vd), go.to(DEV)))
+    assert all(torch.equal(a, b) for a, b in zip(*outs))

@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 import torch
 
+from oracle import attention_oracle as ao
 from oracle.attention_oracle import attention_fwd_oracle, online_softmax_tiles
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "attn_small.npz")
@@ -124,3 +125,28 @@ def test_golden_fixture():
         o, lse = attention_fwd_oracle(q, k, v, causal=causal, softmax_scale=float(z["scale"]))
         assert np.allclose(o.numpy(), z[f"o_{tag}"], atol=1e-5, rtol=1e-5)
         assert np.allclose(lse.numpy(), z[f"lse_{tag}"], atol=1e-5, rtol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 2, 37, 53, 16), (2, 1, 64, 64, 32), (1, 1, 5, 9, 8)])
+def test_backward_closed_form_equals_autograd(shape, causal):
+    # the closed-form gradients against torch.autograd on the forward expression, both in float64
+    B, H, M, N, D = shape
+    g = torch.Generator().manual_seed(M * N)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g, dtype=torch.float64) for n in (M, N, N, M))
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    s = (qa / math.sqrt(D)) @ ka.transpose(-1, -2)
+    if causal:
+        s = s.masked_fill(torch.arange(N)[None, :] > torch.arange(M)[:, None], float("-inf"))
+    o = torch.softmax(s, dim=-1) @ va
+    dq_a, dk_a, dv_a = torch.autograd.grad(o, (qa, ka, va), go)
+    dq, dk, dv = ao.attention_bwd_oracle(q, k, v, go, causal=causal, dtype=torch.float64)
+    for name, a, b in (("dQ", dq, dq_a), ("dK", dk, dk_a), ("dV", dv, dv_a)):
+        assert torch.allclose(a, b, rtol=1e-10, atol=1e-12), f"{name}: max diff {(a - b).abs().max().item():.3e}"
+    # fp32 arithmetic of the same formulas stays within fp32 rounding of the float64 result
+    dq32, dk32, dv32 = ao.attention_bwd_oracle(q.float(), k.float(), v.float(), go.float(), causal=causal)
+    for a, b in ((dq32, dq), (dk32, dk), (dv32, dv)):
+        assert (a.double() - b).abs().max().item() <= 1e-4 * max(1.0, b.abs().max().item())
+    # invariants: a key no query may attend gets zero gradient (causal, keys beyond the last query)
+    if causal and N > M:
+        assert float(dk[:, :, M:].abs().max()) == 0.0 and float(dv[:, :, M:].abs().max()) == 0.0
