@@ -5,7 +5,7 @@
 Prints ONE JSON line. The headline value is the attention forward throughput at B=2 H=16 S=8192 D=128 bf16 causal
 (FLOPs counted as 2*B*H*S^2*D); the fused Lion step over 1,308,622,848 fp32 parameters with bf16 momentum (16 bytes
 per parameter) is reported in the "lion" object of the same line, each with its roofline and a CPU baseline timed on
-this host's cores.
+this host's cores. The attention backward of the same shape is reported in "attn_bwd".
 """
 import argparse
 import json
@@ -83,6 +83,20 @@ def bench_attention(steps, warmup, cpu_baseline):
             "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "flops_per_launch": flops,
         },
         "workload": f"attention fwd B={B} H={H} S={S} D={D} bf16 causal, scale 1/sqrt({D})",
+    }
+    # the backward of the same workload (dQ, dK, dV; three launches), reported beside the headline, not part of it
+    from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided
+
+    go = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev)
+    o_fix, lse_fix = out["o"], out["lse"]
+    bwd_flops = 5.0 * B * H * S * S * D      # causal-halved 10*B*H*S^2*D (five GEMMs; the kernels recompute two more)
+    b_step, b_kernel, b_min = _time_steps(lambda: attn_bwd_strided(q, k, v, o_fix, lse_fix, go, (0, 1, 2, 3), True, scale), steps, warmup)
+    res["bwd"] = {
+        "value": bwd_flops / (b_step * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": b_step,
+        "roofline": {"bound": "mfma", "achieved": bwd_flops / (b_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": bwd_flops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": None,
+                     "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "flops_per_launch": bwd_flops},
+        "workload": "attention bwd (delta + dQ + dK/dV kernels) of the same shape, FLOPs by the five-GEMM count",
     }
     if cpu_baseline:
         # bounded sample: all (batch, head) slices of the same workload through the oracle's fp32 vanilla path on all host
@@ -162,8 +176,10 @@ def bench_lion(steps, warmup, cpu_baseline):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults: the GPU's clocks take a few dozen launches to settle after idling (per-launch time of the attention
+    # kernel wanders by 25 % over the first 30 launches, then stays within 1 %), so the warm-up is longer than usual
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--path", choices=["both", "attn", "lion", "copy"], default="both",
                     help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -207,6 +223,8 @@ def main():
         line["cpu_baseline"] = head["cpu_baseline"]
     if attn is not None and lion is not None:
         line["lion"] = {k: v for k, v in lion.items() if k != "workload"}
+    if attn is not None and "bwd" in attn:
+        line["attn_bwd"] = attn["bwd"]
     print(json.dumps(line))
 
 

@@ -855,12 +855,18 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // ---- epilogue: normalise, write O and LSE
 #pragma unroll
   for (int d = 0; d < DBLK; ++d) mfma_result_fence_a(oacc[d]);
+  // A lane holds 4 consecutive d of one query row per accumulator register group: written straight to memory that is
+  // 8 bytes per lane, 16 per row and instruction. Instead the wave's rows are staged in LDS (the rings are free once
+  // every wave is past its last tile; rows padded by 16 bytes against bank conflicts) and leave as whole 16-byte
+  // pieces, 64 lanes covering four consecutive 256-byte rows per instruction.
+  __syncthreads();
+  constexpr int OROW = ROW_BYTES + 16;
+  FO_LDS char* stage = smem + wave_s * (32 * QB) * OROW;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = l_run[qb] + half_swap(l_run[qb]);
     const float inv = 1.0f / l_tot;
     const int qi = q0w + 32 * qb + l32;
-    T* op = (T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)min(qi, Sq - 1) * prm.os[2];
 #pragma unroll
     for (int db = 0; db < DBLK; ++db) {
       f32x16 t = oacc[db][qb];
@@ -871,12 +877,22 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
         vec4 o4;
 #pragma unroll
         for (int u = 0; u < 4; ++u) o4[u] = (T)(t[rg * 4 + u] * inv);
-        if (qi < Sq) *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
+        *(FO_LDS vec4*)(stage + (32 * qb + l32) * OROW + (32 * db + 8 * rg + 4 * hh) * 2) = o4;
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     if (qi < Sq && prm.lse != nullptr && hh == 0)
       prm.lse[(int64_t)bh * Sq + qi] = (m_run[qb] * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+  }
+  {
+    constexpr int CH = ROW_BYTES / 16;                  // 16-byte pieces per row
+    T* obase = (T*)prm.o + b * prm.os[0] + h * prm.os[1];
+#pragma unroll
+    for (int it = 0; it < 32 * QB * CH / 64; ++it) {
+      const int idx = it * 64 + lane, row = idx / CH, ch = idx % CH;
+      const i32x4 piece = *(FO_LDS const i32x4*)(stage + row * OROW + ch * 16);
+      if (q0w + row < Sq) *(i32x4*)(obase + (int64_t)(q0w + row) * prm.os[2] + ch * 8) = piece;
+    }
   }
   }   // pass
 }
