@@ -37,6 +37,7 @@ struct AttnBwdParams {
   int B, H, Sq, Sk;
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];   // element strides: batch, head, sequence
   float scale, scale_log2e;
+  DropoutParams drop;   // used by the kernels instantiated with dropout only
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -110,7 +111,7 @@ __device__ __forceinline__ typename Ops<T>::vec8 col_frag(FO_LDS const char* til
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool DROP>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int TILE_BYTES = kBwdTile * D * 2;
@@ -188,6 +189,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     // register r of block kb holds key key0 + 32*kb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); dead iff
     // key > q or key >= Sk
     vec8 dsf[4];
+    // dropout (flash_attention_triton.py:524-532,599): dP reaches only the kept probabilities, scaled by 1 / (1 - p_drop)
+    const uint32_t drop_row = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0w + l32)) * (uint32_t)Sk + (uint32_t)key0 : 0u;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int key_base = key0 + 32 * kb + 4 * hh;
@@ -197,7 +200,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
       for (int r = 0; r < 16; ++r) {
         const bool dead = lim > -((r & 3) + 8 * (r >> 2));
         const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -lse2));
-        dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dpacc[kb][r] - delta) * scale);
+        float dp = dpacc[kb][r];
+        if constexpr (DROP) {
+          const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2));
+          dp = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? dp * prm.drop.keep_scale : 0.0f;
+        }
+        dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp - delta) * scale);
       }
     }
     // dQ^T += K^T dS^T : four 16-key steps x DBLK d-blocks
@@ -224,7 +232,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool DROP>
 __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int TILE_BYTES = kBwdTile * D * 2;
@@ -306,6 +314,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
       const int lim = CAUSAL ? key - (q0t + 32 * qb + 4 * hh) : 0;
       const int lim_end = Sq - (q0t + 32 * qb + 4 * hh);
       vec8 pf[2], dsf[2];
+      // dropout index of (first query of this lane's register set, this lane's key); consecutive queries are Sk apart
+      const uint32_t drop_base = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0t + 32 * qb + 4 * hh)) * (uint32_t)Sk + (uint32_t)key : 0u;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 l4 = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * j + 4 * hh);
@@ -315,8 +325,14 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
           const int r = 4 * j + u;
           const bool dead = (u + 8 * j) < lim || (u + 8 * j) >= lim_end;
           const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], c, -l4[u] * kLog2e));
-          pf[r >> 3][r & 7] = (T)p;
-          dsf[r >> 3][r & 7] = (T)(p * (dpacc[r] - d4[u]) * scale);
+          float pd = p, dp = dpacc[r];
+          if constexpr (DROP) {
+            const bool keep = dropout_keep(drop_base + (uint32_t)(u + 8 * j) * (uint32_t)Sk, prm.drop.seed, prm.drop.threshold);
+            pd = keep ? p * prm.drop.keep_scale : 0.0f;       // dV sees the dropped, rescaled probabilities (:551-552)
+            dp = keep ? dp * prm.drop.keep_scale : 0.0f;
+          }
+          pf[r >> 3][r & 7] = (T)pd;
+          dsf[r >> 3][r & 7] = (T)(p * (dp - d4[u]) * scale);
         }
       }
       // dV^T += dO^T P and dK^T += Q^T dS : two 16-query steps x DBLK d-blocks
@@ -347,7 +363,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   }
 }
 
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, bool DROP>
 static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
   const int64_t n_bh = (int64_t)p.B * p.H;
@@ -357,14 +373,14 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   if (g_delta > 0x7FFFFFFFll || g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
   const size_t lds_dq = 4 * (size_t)kBwdTile * D * 2;
   const size_t lds_dkdv = lds_dq + 4 * kBwdTile * sizeof(float);
-  static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL>,
+  static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
-  static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL>,
+  static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
   if (a1 != hipSuccess || a2 != hipSuccess) return FO_ERR_LAUNCH;
   attn_bwd_delta_kernel<T, D><<<(unsigned)g_delta, 256, 0, s>>>(p);
-  attn_bwd_dq_kernel<T, D, CAUSAL><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
-  attn_bwd_dkdv_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
+  attn_bwd_dq_kernel<T, D, CAUSAL, DROP><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
+  attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
   return launch_status();
 }
 
@@ -372,9 +388,10 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
 
 using namespace fo;
 
-extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                           float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
-                           const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream) {
+static int attn_bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                         float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                         const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, float dropout_p,
+                         uint32_t seed, uint64_t rng_offset, void* stream) {
   if (!q || !k || !v || !o || !d_o || !lse || !delta_ws || !dq || !dk || !dv || !strides_host) return FO_ERR_NULL_POINTER;
   for (int t = 0; t < 8; ++t)
     if (!strides_host[t]) return FO_ERR_NULL_POINTER;
@@ -393,6 +410,7 @@ extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const vo
   if (all & 15u) return FO_ERR_MISALIGNED;
   if (((uintptr_t)lse | (uintptr_t)delta_ws) & 3u) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;
+  if (!(dropout_p >= 0.0f) || dropout_p >= 1.0f) return FO_ERR_BAD_SHAPE;
 
   AttnBwdParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse; p.delta = delta_ws; p.dq = dq; p.dk = dk; p.dv = dv;
@@ -403,9 +421,26 @@ extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const vo
   p.scale = softmax_scale;
   p.scale_log2e = softmax_scale * kLog2e;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool c = causal != 0;
-#define FO_BWD(T, DD) (c ? launch_bwd<T, DD, true>(p, s) : launch_bwd<T, DD, false>(p, s))
+  const bool c = causal != 0, drop = dropout_p > 0.0f;
+  p.drop = make_dropout(dropout_p, seed, rng_offset);
+#define FO_BWD(T, DD) (drop ? (c ? launch_bwd<T, DD, true, true>(p, s) : launch_bwd<T, DD, false, true>(p, s)) \
+                            : (c ? launch_bwd<T, DD, true, false>(p, s) : launch_bwd<T, DD, false, false>(p, s)))
   if (dtype == FO_DTYPE_BF16) return D == 128 ? FO_BWD(__bf16, 128) : FO_BWD(__bf16, 64);
   return D == 128 ? FO_BWD(_Float16, 128) : FO_BWD(_Float16, 64);
 #undef FO_BWD
+}
+
+extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                           float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                           const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream) {
+  return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
+                       0.0f, 0u, 0ull, stream);
+}
+
+extern "C" int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                                   float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                                   const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
+                                   float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream) {
+  return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
+                       dropout_p, seed, rng_offset, stream);
 }

@@ -45,6 +45,33 @@ __device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst
 #endif
 }
 
+// Dropout of attention probabilities, as the reference defines it (flash_attention_triton.py:38-50,125,216-219): element
+// (b*H + h, q, key) has the 32-bit index  offset + (b*H + h)*Sq*Sk + q*Sk + key  (all arithmetic modulo 2^32); the index,
+// xored with the seed, goes through an integer hash, and the element is KEPT iff the hash exceeds
+// uint32(fp32(p) * 2^32); kept probabilities are multiplied by 1 / (1 - p). Row sums (and so LSE) use the
+// undropped probabilities.
+struct DropoutParams {
+  uint32_t seed;
+  uint32_t threshold;     // uint32(fp32(p) * fp32(4294967295)), computed on the host
+  uint32_t offset;        // low 32 bits of the generator offset
+  float keep_scale;       // 1 / (1 - p) in fp32; 1 when dropout is off
+};
+__host__ __device__ __forceinline__ bool dropout_keep(uint32_t index, uint32_t seed, uint32_t threshold) {
+  uint32_t a = index ^ seed;
+  a ^= a >> 4;
+  a = (a ^ 0xDEADBEEFu) + (a << 5);
+  a ^= a >> 11;
+  return a > threshold;
+}
+inline DropoutParams make_dropout(float p, uint32_t seed, uint64_t rng_offset) {
+  DropoutParams d;
+  d.seed = seed;
+  d.threshold = (uint32_t)(p * 4294967296.0f);       // fp32 product; fp32(4294967295) is 2^32
+  d.offset = (uint32_t)rng_offset;
+  d.keep_scale = 1.0f / (1.0f - p);
+  return d;
+}
+
 // the same with 4 bytes per lane (LDS receives 256 bytes)
 __device__ __forceinline__ void dma4_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)

@@ -41,11 +41,12 @@ struct AttnParams {
   int64_t qs[3], ks[3], vs[3], os[3];   // element strides: batch, head, sequence
   float scale_log2e;                    // softmax_scale * log2(e)
   int n_qblk;
+  DropoutParams drop;                   // used by the kernels instantiated with dropout only
 };
 
 constexpr float kLazyLog2 = 8.0f;   // how far (in log2 units) a tile maximum may exceed the reference before a rescale
 
-template <typename T, int D, bool CAUSAL, bool LAZY, int DBG>
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false>
 __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int ROW_BYTES = D * 2;
@@ -261,12 +262,18 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const float mc = m_run * c;
     float psum = 0.0f;
     vec8 pf[4];
+    // dropout: 32-bit index of this lane's query row at key 0 of the tile (flash_attention_triton.py:125,217)
+    const uint32_t drop_row = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0w + l32)) * (uint32_t)Sk + (uint32_t)key0 : 0u;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = (DBG & 2) ? sacc[kb][r] : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -mc));
-        psum += p;                                     // summed in fp32 before rounding (flash_attention_triton.py:203)
+        float p = (DBG & 2) ? sacc[kb][r] : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -mc));
+        psum += p;                                     // summed in fp32 before rounding and before dropout (flash_attention_triton.py:203)
+        if constexpr (DROP) {
+          const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2));
+          p = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? p * prm.drop.keep_scale : 0.0f;   // :216-219
+        }
         pf[kb * 2 + (r >> 3)][r & 7] = (T)p;           // rounded to the operand type for P.V (:237)
       }
     l_run += psum;
@@ -909,21 +916,23 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
   return launch_status();
 }
 
-template <typename T, int D, bool CAUSAL, bool LAZY, int DBG>
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false>
 static int launch_one(const AttnParams& p, hipStream_t stream) {
   const size_t lds = 4 * (size_t)kBN * D * 2;
   const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
-  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG><<<grid, kWaves * 64, lds, stream>>>(p);
+  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP><<<grid, kWaves * 64, lds, stream>>>(p);
   return launch_status();
 }
 
 // variant bit 0: 1 = exact (eager) rescale instead of the lazy one. Variants 2..7 are timing ablations that produce
 // WRONG results (bit 1: keep re-using the first tiles instead of copying new ones; bit 2: no exponentials).
 template <typename T, int D>
-static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
+static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
+  // dropout runs on the 128-row kernel
+  if (dropout) return causal ? launch_one<T, D, true, true, 0, true>(p, stream) : launch_one<T, D, false, true, 0, true>(p, stream);
   // default: the wide kernel (eight waves x 32 rows) for head_dim 128, the 128-row kernel for head_dim 64
   // (the wide kernel addresses a head's keys with 32-bit byte offsets)
   // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
@@ -974,10 +983,11 @@ static int launch(const AttnParams& p, bool causal, hipStream_t stream) {
 
 using namespace fo;
 
-extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
-                           int B, int H, int Sq, int Sk, int D,
-                           const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
-                           float softmax_scale, int causal, int dtype, void* stream) {
+static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse,
+                         int B, int H, int Sq, int Sk, int D,
+                         const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                         float softmax_scale, int causal, int dtype, float dropout_p, uint32_t seed, uint64_t rng_offset,
+                         void* stream) {
   if (!q || !k || !v || !o || !qs || !ks || !vs || !os) return FO_ERR_NULL_POINTER;
   if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
   if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
@@ -997,6 +1007,7 @@ extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o,
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15u) return FO_ERR_MISALIGNED;
   if (lse && ((uintptr_t)lse & 3u)) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;   // also rejects NaN
+  if (!(dropout_p >= 0.0f) || dropout_p >= 1.0f) return FO_ERR_BAD_SHAPE;
 
   AttnParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
@@ -1004,7 +1015,24 @@ extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o,
   for (int i = 0; i < 3; ++i) { p.qs[i] = qs[i]; p.ks[i] = ks[i]; p.vs[i] = vs[i]; p.os[i] = os[i]; }
   p.scale_log2e = softmax_scale * 1.4426950408889634f;
   p.n_qblk = (int)n_qblk;
+  const bool drop = dropout_p > 0.0f;
+  p.drop = make_dropout(dropout_p, seed, rng_offset);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FO_DTYPE_BF16) return D == 128 ? launch<__bf16, 128>(p, causal != 0, s) : launch<__bf16, 64>(p, causal != 0, s);
-  return D == 128 ? launch<_Float16, 128>(p, causal != 0, s) : launch<_Float16, 64>(p, causal != 0, s);
+  if (dtype == FO_DTYPE_BF16) return D == 128 ? launch<__bf16, 128>(p, causal != 0, drop, s) : launch<__bf16, 64>(p, causal != 0, drop, s);
+  return D == 128 ? launch<_Float16, 128>(p, causal != 0, drop, s) : launch<_Float16, 64>(p, causal != 0, drop, s);
+}
+
+extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                           int B, int H, int Sq, int Sk, int D,
+                           const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                           float softmax_scale, int causal, int dtype, void* stream) {
+  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, 0.0f, 0u, 0ull, stream);
+}
+
+extern "C" int fo_attn_fwd_dropout(const void* q, const void* k, const void* v, void* o, float* lse,
+                                   int B, int H, int Sq, int Sk, int D,
+                                   const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                                   float softmax_scale, int causal, int dtype, float dropout_p, uint32_t seed, uint64_t rng_offset,
+                                   void* stream) {
+  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, dropout_p, seed, rng_offset, stream);
 }

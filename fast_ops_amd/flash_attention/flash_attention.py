@@ -18,6 +18,7 @@ import ctypes
 import math
 from typing import Optional, Tuple, Union
 
+import numpy as np
 import torch
 from torch import Tensor
 from torch.autograd import Function
@@ -42,11 +43,27 @@ def _check_inputs(q: Tensor, k: Tensor, v: Tensor) -> None:
         raise RuntimeError("The last dimension of Q, K and V must be contiguous")
 
 
+Dropout = Tuple[float, int, int]   # (dropout_p, seed, generator offset)
+
+
+def next_dropout_state(n_elements: int) -> Tuple[int, int]:
+    """(seed, offset) for a dropout mask over ``n_elements`` attention probabilities, taken from torch's generator of the
+    current device, whose offset is advanced past them: what increment_philox_state does in the reference
+    (flash_attention_triton.py:641-665). The last 16 bytes of the generator state are (seed, offset) as two uint64."""
+    state = torch.cuda.get_rng_state()
+    words = state.numpy().view(np.uint64)
+    seed, offset = int(words[-2]), int(words[-1])
+    words[-1] = np.uint64((offset + 4 * math.ceil(n_elements / 4)) % (1 << 64))
+    torch.cuda.set_rng_state(state)
+    return seed, offset
+
+
 def attn_fwd_strided(
-    q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int], causal: bool, softmax_scale: Optional[float]
+    q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int], causal: bool, softmax_scale: Optional[float],
+    dropout: Optional[Dropout] = None,
 ) -> Tuple[Tensor, Tensor]:
-    """Launches fo_attn_fwd. ``dims`` = positions of (batch, head, sequence, head_dim) in the tensors' shapes.
-    Returns (O with q's shape, dtype and layout; LSE fp32 [B, H, Sq])."""
+    """Launches fo_attn_fwd (fo_attn_fwd_dropout when ``dropout`` is given). ``dims`` = positions of (batch, head,
+    sequence, head_dim) in the tensors' shapes. Returns (O with q's shape, dtype and layout; LSE fp32 [B, H, Sq])."""
     _check_inputs(q, k, v)
     ib, ih, is_, id_ = dims
     B, H, Sq, D = q.shape[ib], q.shape[ih], q.shape[is_], q.shape[id_]
@@ -64,7 +81,7 @@ def attn_fwd_strided(
         # columns of V only produce output columns that are dropped; the scale stays that of the true head_dim.
         Dp = 64 if D < 64 else 128
         pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
-        o_p, lse = attn_fwd_strided(pad(q), pad(k), pad(v), dims, causal, scale)
+        o_p, lse = attn_fwd_strided(pad(q), pad(k), pad(v), dims, causal, scale, dropout)
         o = torch.empty_like(q)
         o.copy_(o_p.narrow(id_, 0, D))
         return o, lse
@@ -75,18 +92,20 @@ def attn_fwd_strided(
     strides = lambda t: _I64x3(t.stride(ib), t.stride(ih), t.stride(is_))
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        status = _lib.load().fo_attn_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
-            B, H, Sq, Sk, D, strides(q), strides(k), strides(v), strides(o),
-            scale, int(bool(causal)), _DTYPE_CODE[q.dtype], stream,
-        )
+        args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                B, H, Sq, Sk, D, strides(q), strides(k), strides(v), strides(o),
+                scale, int(bool(causal)), _DTYPE_CODE[q.dtype])
+        if dropout is None or dropout[0] == 0.0:
+            status = _lib.load().fo_attn_fwd(*args, stream)
+        else:
+            status = _lib.load().fo_attn_fwd_dropout(*args, float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64), stream)
     _lib.check(status, "fo_attn_fwd")
     return o, lse
 
 
 def attn_bwd_strided(
     q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor, d_o: Tensor, dims: Tuple[int, int, int, int], causal: bool,
-    softmax_scale: Optional[float],
+    softmax_scale: Optional[float], dropout: Optional[Dropout] = None,
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """Launches fo_attn_bwd. Returns (dQ, dK, dV) with the shapes and dtypes of q, k, v (dense; a K/V whose heads are
     an expanded view gets a full-size gradient, which autograd then reduces)."""
@@ -101,7 +120,7 @@ def attn_bwd_strided(
         # same zero padding as the forward; O's padded columns are zero, so delta and the padded gradient columns are too
         Dp = 64 if D < 64 else 128
         pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
-        dq, dk, dv = attn_bwd_strided(pad(q), pad(k), pad(v), pad(o), lse, pad(d_o), dims, causal, scale)
+        dq, dk, dv = attn_bwd_strided(pad(q), pad(k), pad(v), pad(o), lse, pad(d_o), dims, causal, scale, dropout)
         return tuple(t.narrow(id_, 0, D).contiguous() for t in (dq, dk, dv))
     if d_o.stride(-1) != 1 or any(s % 8 for s in d_o.stride()[:-1]):
         d_o = d_o.contiguous()
@@ -117,11 +136,12 @@ def attn_bwd_strided(
     ptrs = (ctypes.POINTER(ctypes.c_int64) * 8)(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in arrays])
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        status = _lib.load().fo_attn_bwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, Sq, Sk, D, ptrs, scale, int(bool(causal)),
-            _DTYPE_CODE[q.dtype], stream,
-        )
+        args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, Sq, Sk, D, ptrs, scale, int(bool(causal)), _DTYPE_CODE[q.dtype])
+        if dropout is None or dropout[0] == 0.0:
+            status = _lib.load().fo_attn_bwd(*args, stream)
+        else:
+            status = _lib.load().fo_attn_bwd_dropout(*args, float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64), stream)
     _lib.check(status, "fo_attn_bwd")
     return dq, dk, dv
 
@@ -129,17 +149,18 @@ def attn_bwd_strided(
 class FlashAttentionFunction(Function):
     @staticmethod
     def forward(ctx, Q: Tensor, K: Tensor, V: Tensor, causal: bool = False, softmax_scale: Optional[float] = None,
-                return_lse: bool = False):
+                return_lse: bool = False, dropout: Optional[Dropout] = None):
         """
         :param Q: (B, H, M, D) Query tensor.
         :param K: (B, H, N, D) Key tensor.
         :param V: (B, H, N, D) Value tensor.
         :returns: (B, H, M, D), and the (B, H, M) fp32 logsumexp when ``return_lse``
         """
-        o, lse = attn_fwd_strided(Q, K, V, (0, 1, 2, 3), causal, softmax_scale)
+        o, lse = attn_fwd_strided(Q, K, V, (0, 1, 2, 3), causal, softmax_scale, dropout)
         ctx.save_for_backward(Q, K, V, o, lse)   # what a backward pass needs (flash_attention_triton.py:826)
         ctx.causal = causal
         ctx.softmax_scale = softmax_scale
+        ctx.dropout = dropout                    # (p, seed, offset): the backward regenerates the mask (:824-828)
         if return_lse:
             ctx.mark_non_differentiable(lse)
             return o, lse
@@ -150,19 +171,21 @@ class FlashAttentionFunction(Function):
         """:param dO: (B, H, M, D) Output gradient. The reference leaves this unimplemented (flash_attention.py:40-45);
         here it is what the reference's Triton backward computes (flash_attention_triton.py:832-958)."""
         Q, K, V, o, lse = ctx.saved_tensors
-        dq, dk, dv = attn_bwd_strided(Q, K, V, o, lse, dO, (0, 1, 2, 3), ctx.causal, ctx.softmax_scale)
-        return dq, dk, dv, None, None, None
+        dq, dk, dv = attn_bwd_strided(Q, K, V, o, lse, dO, (0, 1, 2, 3), ctx.causal, ctx.softmax_scale, ctx.dropout)
+        return dq, dk, dv, None, None, None, None
 
 
 class _FlashAttnBSHD(Function):
     """flash_attn's autograd node: the same kernels on [batch, seqlen, nheads, headdim] tensors."""
 
     @staticmethod
-    def forward(ctx, q: Tensor, k: Tensor, v: Tensor, causal: bool, softmax_scale: Optional[float], return_lse: bool):
-        o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale)
+    def forward(ctx, q: Tensor, k: Tensor, v: Tensor, causal: bool, softmax_scale: Optional[float], return_lse: bool,
+                dropout: Optional[Dropout]):
+        o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale, dropout)
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.causal = causal
         ctx.softmax_scale = softmax_scale
+        ctx.dropout = dropout
         if return_lse:
             ctx.mark_non_differentiable(lse)
             return o, lse
@@ -171,12 +194,22 @@ class _FlashAttnBSHD(Function):
     @staticmethod
     def backward(ctx, dO: Tensor, *unused):
         q, k, v, o, lse = ctx.saved_tensors
-        dq, dk, dv = attn_bwd_strided(q, k, v, o, lse, dO, (0, 2, 1, 3), ctx.causal, ctx.softmax_scale)
-        return dq, dk, dv, None, None, None
+        dq, dk, dv = attn_bwd_strided(q, k, v, o, lse, dO, (0, 2, 1, 3), ctx.causal, ctx.softmax_scale, ctx.dropout)
+        return dq, dk, dv, None, None, None, None
+
+
+def _dropout_arg(dropout_p: float, dropout_state: Optional[Tuple[int, int]], n_elements: int) -> Optional[Dropout]:
+    if dropout_p == 0.0:
+        return None
+    if not 0.0 <= dropout_p < 1.0:
+        raise RuntimeError(f"dropout_p must be in [0, 1), got {dropout_p}")
+    seed, offset = dropout_state if dropout_state is not None else next_dropout_state(n_elements)
+    return (float(dropout_p), int(seed), int(offset))
 
 
 def multi_head_attention(
-    Q: Tensor, K: Tensor, V: Tensor, *, causal: bool = False, softmax_scale: Optional[float] = None, return_lse: bool = False
+    Q: Tensor, K: Tensor, V: Tensor, *, causal: bool = False, softmax_scale: Optional[float] = None, return_lse: bool = False,
+    dropout_p: float = 0.0, dropout_state: Optional[Tuple[int, int]] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """FlashAttention forward (https://arxiv.org/abs/2205.14135), B = batch, H = heads, M = queries, N = keys, D = head dim.
 
@@ -190,19 +223,21 @@ def multi_head_attention(
     :param causal: query i attends keys j <= i
     :param softmax_scale: multiplier of Q K^T, default 1/sqrt(D)
     :param return_lse: also return the (B, H, M) fp32 logsumexp of the scaled scores
+    :param dropout_p: probability of dropping an attention probability (flash_attention_triton.py:216-219)
+    :param dropout_state: (seed, offset) of the mask; default: taken from torch's generator, which is advanced
     :returns: (B, H, M, D)
     """
-    return FlashAttentionFunction.apply(Q, K, V, causal, softmax_scale, return_lse)
+    drop = _dropout_arg(dropout_p, dropout_state, Q.shape[0] * Q.shape[1] * Q.shape[2] * K.shape[2])
+    return FlashAttentionFunction.apply(Q, K, V, causal, softmax_scale, return_lse, drop)
 
 
 def flash_attn(
     q: Tensor, k: Tensor, v: Tensor, bias: Optional[Tensor] = None, causal: bool = False, dropout_p: float = 0.0,
-    softmax_scale: Optional[float] = None, return_lse: bool = False,
+    softmax_scale: Optional[float] = None, return_lse: bool = False, dropout_state: Optional[Tuple[int, int]] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """The [batch, seqlen, nheads, headdim] surface of flash_attn_triton (flash_attention_triton.py:722-737,961),
-    differentiable. Bias and dropout are not implemented and raise."""
+    differentiable, with dropout. Bias is not implemented and raises."""
     if bias is not None:
         raise RuntimeError("attention bias is not implemented")
-    if dropout_p != 0.0:
-        raise RuntimeError("attention dropout is not implemented")
-    return _FlashAttnBSHD.apply(q, k, v, causal, softmax_scale, return_lse)
+    drop = _dropout_arg(dropout_p, dropout_state, q.shape[0] * q.shape[2] * q.shape[1] * k.shape[1])
+    return _FlashAttnBSHD.apply(q, k, v, causal, softmax_scale, return_lse, drop)

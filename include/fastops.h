@@ -98,6 +98,26 @@ int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, cons
                 const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * The same two with dropout of the attention probabilities, as the reference's Triton kernels define it
+ * (flash_attention_triton.py:38-50 hash, :125,:216-219 forward, :421,:524-532,:551,:599 backward): element
+ * (b*H + h, q, key) has the 32-bit index rng_offset + (b*H + h)*Sq*Sk + q*Sk + key (arithmetic modulo 2^32); the index
+ * xor seed goes through the integer hash of :44-48; the probability is kept iff the hash exceeds
+ * uint32(fp32(dropout_p) * 2^32) and is then multiplied by 1 / (1 - dropout_p). Row sums, and so LSE, use the undropped
+ * probabilities. The caller supplies seed and offset (the reference takes them from torch's generator state,
+ * :641-665) and must pass the same pair to the backward. dropout_p in [0, 1); 0 is exactly fo_attn_fwd / fo_attn_bwd.
+ */
+int fo_attn_fwd_dropout(const void* q, const void* k, const void* v, void* o, float* lse,
+                        int B, int H, int Sq, int Sk, int D,
+                        const int64_t* q_strides_host, const int64_t* k_strides_host,
+                        const int64_t* v_strides_host, const int64_t* o_strides_host,
+                        float softmax_scale, int causal, int dtype,
+                        float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream);
+int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                        float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                        const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
+                        float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * Fused Lion step: fp32 parameters, fp32 gradients, bf16 momentum, one pass.
  * Per element, in this order and with these rounding points (lion_optimizer_ref.py:51,64,65,67):
  *     p1 = p * c_wd

@@ -30,6 +30,21 @@ import numpy as np
 import torch
 
 
+def dropout_keep_mask(dropout_p: float, seed: int, rng_offset: int, B: int, H: int, M: int, N: int) -> np.ndarray:
+    """The reference's dropout mask (flash_attention_triton.py:38-50 hash, :125,:216-217 / :682-691 indices): bool
+    [B, H, M, N], True = kept. Index of (b, h, m, n) = rng_offset + (b*H + h)*M*N + m*N + n in 32-bit arithmetic;
+    a = index ^ seed;  a ^= a >> 4;  a = (a ^ 0xDEADBEEF) + (a << 5);  a ^= a >> 11;  keep = a > uint32(fp32(p) * fp32(2^32 - 1)).
+    Pinned by tests/test_oracle_attention.py: a pure-Python-integer restatement on small shapes, hand-computed hashes,
+    the kept fraction, and independence of offset-shifted masks."""
+    idx = (np.arange(B * H * M * N, dtype=np.uint64) + np.uint64(rng_offset % (1 << 32))).astype(np.uint32)
+    a = idx ^ np.uint32(seed & 0xFFFFFFFF)
+    a = a ^ (a >> np.uint32(4))
+    a = ((a ^ np.uint32(0xDEADBEEF)).astype(np.uint64) + (a.astype(np.uint64) << np.uint64(5))).astype(np.uint32)
+    a = a ^ (a >> np.uint32(11))
+    thr = np.uint32(int(np.float32(dropout_p) * np.float32(4294967295)))
+    return (a > thr).reshape(B, H, M, N)
+
+
 def attention_fwd_oracle(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -37,6 +52,7 @@ def attention_fwd_oracle(
     causal: bool = False,
     softmax_scale: Optional[float] = None,
     q_chunk: int = 1024,
+    dropout: Optional[Tuple[float, int, int]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """fp32 softmax(scale * Q K^T + mask) V and its logsumexp. Returns (O fp32 [B,H,M,D], LSE fp32 [B,H,M]).
 
@@ -50,6 +66,12 @@ def attention_fwd_oracle(
     qf, kf, vf = q.float().cpu(), k.float().cpu(), v.float().cpu()   # attention_ref.py:41-43
     out = torch.empty(B, H, M, D, dtype=torch.float32)
     lse = torch.empty(B, H, M, dtype=torch.float32)
+    keep = None
+    if dropout is not None and dropout[0] > 0.0:
+        # dropout of the probabilities after the row sums are taken (flash_attention_triton.py:203,216-219): LSE is that
+        # of the undropped scores, kept probabilities are scaled by 1 / (1 - p) computed in fp32
+        keep = torch.from_numpy(dropout_keep_mask(dropout[0], dropout[1], dropout[2], B, H, M, N))
+        keep_scale = float(np.float32(1.0) / (np.float32(1.0) - np.float32(dropout[0])))
     for b in range(B):
         for h in range(H):
             kt = kf[b, h].t()
@@ -62,6 +84,8 @@ def attention_fwd_oracle(
                     scores = scores.masked_fill(cols > rows, float("-inf"))  # attention_ref.py:54-58 (triu, diagonal=1)
                 lse[b, h, m0:m1] = torch.logsumexp(scores, dim=-1)
                 attn = torch.softmax(scores, dim=-1)                          # attention_ref.py:59
+                if keep is not None:
+                    attn = torch.where(keep[b, h, m0:m1], attn * keep_scale, torch.zeros_like(attn))
                 out[b, h, m0:m1] = attn @ vf[b, h]                            # attention_ref.py:67
     return out, lse
 
@@ -74,6 +98,7 @@ def attention_bwd_oracle(
     causal: bool = False,
     softmax_scale: Optional[float] = None,
     dtype: torch.dtype = torch.float32,
+    dropout: Optional[Tuple[float, int, int]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of sum(O * dO) with respect to Q, K, V, in closed form, one (batch, head) at a time:
 
@@ -82,13 +107,19 @@ def attention_bwd_oracle(
 
     which is what the reference's backward computes tile by tile (flash_attention_triton.py:273-315 delta pre-pass,
     :497-578 per-tile dv / dp / ds / dk / dq) and what autograd gives for attention_ref.py:41-67. ``dtype`` is the
-    arithmetic type (fp32 for the oracle proper, float64 to pin it). Returns (dQ, dK, dV) in ``dtype`` on the CPU.
+    arithmetic type (fp32 for the oracle proper, float64 to pin it). With dropout (mask Z = keep / (1 - p), :524-532,
+    :551,:599): O = (P * Z) V, dV = (P * Z)^T dO, dP = (dO V^T) * Z, the rest unchanged.
+    Returns (dQ, dK, dV) in ``dtype`` on the CPU.
     Pinned by tests/test_oracle_attention.py against torch.autograd on the forward expression in float64."""
     B, H, M, D = q.shape
     N = k.shape[2]
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
     qf, kf, vf, gf = (t.to(dtype).cpu() for t in (q, k, v, d_o))
     dq, dk, dv = torch.zeros_like(qf), torch.zeros_like(kf), torch.zeros_like(vf)
+    z = None
+    if dropout is not None and dropout[0] > 0.0:
+        keep = torch.from_numpy(dropout_keep_mask(dropout[0], dropout[1], dropout[2], B, H, M, N))
+        z = keep.to(dtype) * float(np.float32(1.0) / (np.float32(1.0) - np.float32(dropout[0])))
     for b in range(B):
         for h in range(H):
             s = (qf[b, h] * scale) @ kf[b, h].t()
@@ -97,9 +128,12 @@ def attention_bwd_oracle(
                 cols = torch.arange(N).unsqueeze(0)
                 s = s.masked_fill(cols > rows, float("-inf"))
             p = torch.softmax(s, dim=-1)
-            o = p @ vf[b, h]
-            dv[b, h] = p.t() @ gf[b, h]
+            pz = p if z is None else p * z[b, h]
+            o = pz @ vf[b, h]
+            dv[b, h] = pz.t() @ gf[b, h]
             dp = gf[b, h] @ vf[b, h].t()
+            if z is not None:
+                dp = dp * z[b, h]
             delta = (gf[b, h] * o).sum(dim=-1, keepdim=True)
             ds = p * (dp - delta)
             dq[b, h] = (ds @ kf[b, h]) * scale

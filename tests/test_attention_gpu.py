@@ -172,8 +172,8 @@ def test_bshd_surface_and_multi_query(kernel_variant):
     _check(o.transpose(1, 2), lse, o_ref, lse_ref, "BSHD multi-query")
     with pytest.raises(RuntimeError, match="bias"):
         flash_attn(qd, kd, vd, bias=torch.zeros(1, device=DEV))
-    with pytest.raises(RuntimeError, match="dropout"):
-        flash_attn(qd, kd, vd, dropout_p=0.1)
+    with pytest.raises(RuntimeError, match="dropout_p"):
+        flash_attn(qd, kd, vd, dropout_p=1.5)
 
 
 @pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)

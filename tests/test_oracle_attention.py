@@ -150,3 +150,67 @@ def test_backward_closed_form_equals_autograd(shape, causal):
     # invariants: a key no query may attend gets zero gradient (causal, keys beyond the last query)
     if causal and N > M:
         assert float(dk[:, :, M:].abs().max()) == 0.0 and float(dv[:, :, M:].abs().max()) == 0.0
+
+
+def _hash_python(index, seed):
+    a = (index ^ seed) & 0xFFFFFFFF
+    a ^= a >> 4
+    a = ((a ^ 0xDEADBEEF) + ((a << 5) & 0xFFFFFFFF)) & 0xFFFFFFFF
+    a ^= a >> 11
+    return a
+
+
+def test_dropout_mask_restatements_and_statistics():
+    # (1) numpy restatement == pure-Python-integer restatement, including 32-bit wrap of the index
+    B, H, M, N, p, seed, off = 2, 3, 5, 7, 0.3, 0x12345678, (1 << 32) - 50
+    mask = ao.dropout_keep_mask(p, seed, off, B, H, M, N)
+    thr = int(np.float32(p) * np.float32(4294967295))
+    for b in range(B):
+        for h in range(H):
+            for m in range(M):
+                for n in range(N):
+                    idx = (off + (b * H + h) * M * N + m * N + n) & 0xFFFFFFFF
+                    assert bool(mask[b, h, m, n]) == (_hash_python(idx, seed) > thr)
+    # (2) the hash on inputs worked out by hand: a = 0 -> 0 ^ 0 = 0; (0 ^ 0xDEADBEEF) + 0 = 0xDEADBEEF;
+    #     0xDEADBEEF ^ (0xDEADBEEF >> 11) = 0xDEADBEEF ^ 0x001BD5B7 = 0xDEB66B58
+    assert _hash_python(0, 0) == 0xDEB66B58
+    #     a = 16: 16 ^ 1 = 17; (17 ^ 0xDEADBEEF) + (17 << 5) = 0xDEADBEFE + 0x220 = 0xDEADC11E; ^ (>> 11 = 0x001BD5B8) = 0xDEB614A6
+    assert _hash_python(16, 0) == 0xDEB614A6
+    # (3) threshold: p = 0 keeps everything whose hash is non-zero, p -> 1 keeps nothing
+    assert ao.dropout_keep_mask(0.0, 1, 0, 1, 1, 64, 64).mean() > 0.999
+    assert ao.dropout_keep_mask(0.999999, 1, 0, 1, 1, 64, 64).mean() < 1e-3
+    # (4) statistics, in the reference's own style (tests/test_flash_attention_triton.py:176-280 accumulates keeps over
+    #     1000 calls with advancing offsets): averaged over offsets that span the 32-bit index range the kept fraction
+    #     is 1 - p. (Within ONE mask of fewer than 2^22 elements the hash is far from uniform - its top bits depend only
+    #     on index bits 22 and up - so a single mask is almost entirely kept or almost entirely dropped; that is the
+    #     reference's definition and is reproduced as it is.)
+    for p in (0.1, 0.17, 0.5):
+        for seed in (0, 123, 0xDEADBEEF):
+            fracs = [ao.dropout_keep_mask(p, seed, off, 1, 1, 64, 64).mean() for off in range(0, 1 << 32, 1 << 23)]
+            assert abs(np.mean(fracs) - (1 - p)) < 1.5e-2, (p, seed, np.mean(fracs))
+    # shifting the offset by the mask's size gives the continuation of the same index stream
+    a = ao.dropout_keep_mask(0.2, 5, 0, 1, 2, 8, 16)
+    b = ao.dropout_keep_mask(0.2, 5, 8 * 16, 1, 1, 8, 16)
+    assert np.array_equal(a[0, 1], b[0, 0])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_backward_with_dropout_equals_autograd(causal):
+    B, H, M, N, D = 1, 2, 33, 41, 16
+    drop = (0.25, 99, 1000)
+    g = torch.Generator().manual_seed(5)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g, dtype=torch.float64) for n in (M, N, N, M))
+    z = torch.from_numpy(ao.dropout_keep_mask(*drop, B, H, M, N)).double() * float(np.float32(1.0) / (np.float32(1.0) - np.float32(drop[0])))
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    s = (qa / math.sqrt(D)) @ ka.transpose(-1, -2)
+    if causal:
+        s = s.masked_fill(torch.arange(N)[None, :] > torch.arange(M)[:, None], float("-inf"))
+    o = (torch.softmax(s, dim=-1) * z) @ va
+    ref = torch.autograd.grad(o, (qa, ka, va), go)
+    got = ao.attention_bwd_oracle(q, k, v, go, causal=causal, dtype=torch.float64, dropout=drop)
+    for a, b in zip(got, ref):
+        assert torch.allclose(a, b, rtol=1e-10, atol=1e-12)
+    o32, lse32 = attention_fwd_oracle(q.float(), k.float(), v.float(), causal=causal, dropout=drop)
+    assert torch.allclose(o32.double(), o.detach(), rtol=1e-4, atol=1e-5)
+    # LSE is that of the undropped scores
+    assert torch.allclose(lse32.double(), torch.logsumexp(s.detach(), dim=-1), rtol=1e-5, atol=1e-5)
