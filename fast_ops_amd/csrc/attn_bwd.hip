@@ -38,6 +38,7 @@ struct AttnBwdParams {
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];   // element strides: batch, head, sequence
   float scale, scale_log2e;
   DropoutParams drop;   // used by the kernels instantiated with dropout only
+  BiasParams bias;      // used by the kernels instantiated with bias only
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -111,7 +112,7 @@ __device__ __forceinline__ typename Ops<T>::vec8 col_frag(FO_LDS const char* til
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, bool CAUSAL, bool DROP>
+template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int TILE_BYTES = kBwdTile * D * 2;
@@ -191,6 +192,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     vec8 dsf[4];
     // dropout (flash_attention_triton.py:524-532,599): dP reaches only the kept probabilities, scaled by 1 / (1 - p_drop)
     const uint32_t drop_row = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0w + l32)) * (uint32_t)Sk + (uint32_t)key0 : 0u;
+    // bias row of this lane's query (flash_attention_triton.py:497-509); keys past the end re-read the last one
+    const int64_t bias_row = BIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)qrow * prm.bias.strides[2] : 0;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int key_base = key0 + 32 * kb + 4 * hh;
@@ -199,7 +202,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const bool dead = lim > -((r & 3) + 8 * (r >> 2));
-        const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, -lse2));
+        float shift = -lse2;
+        if constexpr (BIAS) shift = __builtin_fmaf(load_bias<T>(prm.bias, bias_row + min(key_base + (r & 3) + 8 * (r >> 2), Sk - 1)), kLog2e, -lse2);
+        const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, shift));
         float dp = dpacc[kb][r];
         if constexpr (DROP) {
           const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2));
@@ -232,7 +237,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, bool CAUSAL, bool DROP>
+template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
 __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int TILE_BYTES = kBwdTile * D * 2;
@@ -316,6 +321,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
       vec8 pf[2], dsf[2];
       // dropout index of (first query of this lane's register set, this lane's key); consecutive queries are Sk apart
       const uint32_t drop_base = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0t + 32 * qb + 4 * hh)) * (uint32_t)Sk + (uint32_t)key : 0u;
+      // bias column of this lane's key; queries past the end re-read the last one
+      const int64_t bias_col = BIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] + krow : 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 l4 = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * j + 4 * hh);
@@ -324,7 +331,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
         for (int u = 0; u < 4; ++u) {
           const int r = 4 * j + u;
           const bool dead = (u + 8 * j) < lim || (u + 8 * j) >= lim_end;
-          const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], c, -l4[u] * kLog2e));
+          float shift = -l4[u] * kLog2e;
+          if constexpr (BIAS) {
+            const int qi = min(q0t + 32 * qb + 4 * hh + u + 8 * j, Sq - 1);
+            shift = __builtin_fmaf(load_bias<T>(prm.bias, bias_col + (int64_t)qi * prm.bias.strides[2]), kLog2e, shift);
+          }
+          const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], c, shift));
           float pd = p, dp = dpacc[r];
           if constexpr (DROP) {
             const bool keep = dropout_keep(drop_base + (uint32_t)(u + 8 * j) * (uint32_t)Sk, prm.drop.seed, prm.drop.threshold);
@@ -363,7 +375,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   }
 }
 
-template <typename T, int D, bool CAUSAL, bool DROP>
+template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
 static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
   const int64_t n_bh = (int64_t)p.B * p.H;
@@ -373,14 +385,14 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   if (g_delta > 0x7FFFFFFFll || g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
   const size_t lds_dq = 4 * (size_t)kBwdTile * D * 2;
   const size_t lds_dkdv = lds_dq + 4 * kBwdTile * sizeof(float);
-  static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP>,
+  static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
-  static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP>,
+  static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
   if (a1 != hipSuccess || a2 != hipSuccess) return FO_ERR_LAUNCH;
   attn_bwd_delta_kernel<T, D><<<(unsigned)g_delta, 256, 0, s>>>(p);
-  attn_bwd_dq_kernel<T, D, CAUSAL, DROP><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
-  attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
+  attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
+  attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
   return launch_status();
 }
 
@@ -391,7 +403,8 @@ using namespace fo;
 static int attn_bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                          float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
                          const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, float dropout_p,
-                         uint32_t seed, uint64_t rng_offset, void* stream) {
+                         uint32_t seed, uint64_t rng_offset, const void* bias, const int64_t* bias_strides, int bias_dtype,
+                         void* stream) {
   if (!q || !k || !v || !o || !d_o || !lse || !delta_ws || !dq || !dk || !dv || !strides_host) return FO_ERR_NULL_POINTER;
   for (int t = 0; t < 8; ++t)
     if (!strides_host[t]) return FO_ERR_NULL_POINTER;
@@ -411,6 +424,12 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   if (((uintptr_t)lse | (uintptr_t)delta_ws) & 3u) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;
   if (!(dropout_p >= 0.0f) || dropout_p >= 1.0f) return FO_ERR_BAD_SHAPE;
+  if (bias) {
+    if (!bias_strides) return FO_ERR_NULL_POINTER;
+    if (bias_dtype != FO_DTYPE_F32 && bias_dtype != dtype) return FO_ERR_BAD_DTYPE;
+    if (bias_strides[0] < 0 || bias_strides[1] < 0 || bias_strides[2] < 0) return FO_ERR_BAD_STRIDE;
+    if ((uintptr_t)bias & (bias_dtype == FO_DTYPE_F32 ? 3u : 1u)) return FO_ERR_MISALIGNED;
+  }
 
   AttnBwdParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse; p.delta = delta_ws; p.dq = dq; p.dk = dk; p.dv = dv;
@@ -423,18 +442,23 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool c = causal != 0, drop = dropout_p > 0.0f;
   p.drop = make_dropout(dropout_p, seed, rng_offset);
-#define FO_BWD(T, DD) (drop ? (c ? launch_bwd<T, DD, true, true>(p, s) : launch_bwd<T, DD, false, true>(p, s)) \
-                            : (c ? launch_bwd<T, DD, true, false>(p, s) : launch_bwd<T, DD, false, false>(p, s)))
+  p.bias.ptr = bias;
+  for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
+  p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
+#define FO_BWD2(T, DD, BI) (drop ? (c ? launch_bwd<T, DD, true, true, BI>(p, s) : launch_bwd<T, DD, false, true, BI>(p, s)) \
+                                 : (c ? launch_bwd<T, DD, true, false, BI>(p, s) : launch_bwd<T, DD, false, false, BI>(p, s)))
+#define FO_BWD(T, DD) (bias ? FO_BWD2(T, DD, true) : FO_BWD2(T, DD, false))
   if (dtype == FO_DTYPE_BF16) return D == 128 ? FO_BWD(__bf16, 128) : FO_BWD(__bf16, 64);
   return D == 128 ? FO_BWD(_Float16, 128) : FO_BWD(_Float16, 64);
 #undef FO_BWD
+#undef FO_BWD2
 }
 
 extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                            float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
                            const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream) {
   return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
-                       0.0f, 0u, 0ull, stream);
+                       0.0f, 0u, 0ull, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
@@ -442,5 +466,17 @@ extern "C" int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, 
                                    const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
                                    float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream) {
   return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
-                       dropout_p, seed, rng_offset, stream);
+                       dropout_p, seed, rng_offset, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int fo_attn_bwd_ex(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                              float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                              const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
+                              const fo_attn_extras* extras, void* stream) {
+  if (!extras)
+    return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
+                         0.0f, 0u, 0ull, nullptr, nullptr, 0, stream);
+  return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
+                       extras->dropout_p, extras->dropout_seed, extras->dropout_offset, extras->bias, extras->bias_strides,
+                       extras->bias_dtype, stream);
 }

@@ -72,6 +72,19 @@ inline DropoutParams make_dropout(float p, uint32_t seed, uint64_t rng_offset) {
   return d;
 }
 
+// Additive bias on the scaled scores (flash_attention_triton.py:176-198, attention_ref.py:50-51): element
+// (b, h, q, key) at bias + b*strides[0] + h*strides[1] + q*strides[2] + key, a stride of 0 broadcasting that dimension
+// (the reference's "vector" bias is strides[2] == 0); fp32 or the operand type.
+struct BiasParams {
+  const void* ptr;
+  int64_t strides[3];
+  int is_f32;
+};
+template <typename T>
+__device__ __forceinline__ float load_bias(const BiasParams& bp, int64_t at) {
+  return bp.is_f32 ? ((const float*)bp.ptr)[at] : (float)((const T*)bp.ptr)[at];
+}
+
 // the same with 4 bytes per lane (LDS receives 256 bytes)
 __device__ __forceinline__ void dma4_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)

@@ -42,11 +42,12 @@ struct AttnParams {
   float scale_log2e;                    // softmax_scale * log2(e)
   int n_qblk;
   DropoutParams drop;                   // used by the kernels instantiated with dropout only
+  BiasParams bias;                      // used by the kernels instantiated with bias only
 };
 
 constexpr float kLazyLog2 = 8.0f;   // how far (in log2 units) a tile maximum may exceed the reference before a rescale
 
-template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false>
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false>
 __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int ROW_BYTES = D * 2;
@@ -168,7 +169,9 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.0f;
   float m_run = -INFINITY;   // reference maximum (raw, unscaled scores) of this lane's query row
   float l_run = 0.0f;        // running sum of this lane's half of the keys
-  const float c = prm.scale_log2e;
+  // with a bias the scores are turned into base-2 logits (score * scale * log2e + bias * log2e) right after the mask, and
+  // everything downstream sees a scale of 1
+  const float c = BIAS ? 1.0f : prm.scale_log2e;
 
   // per-lane LDS read offsets that do not depend on the tile
   //  K (ds_read_b128): row = 32*kb + l32, logical chunk = 2*ks + hh
@@ -237,6 +240,18 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
       }
     }
 
+    if constexpr (BIAS) {
+      // qk * softmax_scale + bias (flash_attention_triton.py:198); rows and keys past the end re-read the last ones
+      const int64_t brow = b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)min(q0w + l32, Sq - 1) * prm.bias.strides[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = min(key0 + 32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2), Sk - 1);
+          sacc[kb][r] = __builtin_fmaf(sacc[kb][r], prm.scale_log2e, load_bias<T>(prm.bias, brow + key) * 1.4426950408889634f);
+        }
+    }
+
     // ---- online softmax (base-2 domain) with a lazily updated reference maximum.
     // exp2 is taken relative to m_run, which is only raised (and O, l rescaled) when some row's tile maximum exceeds it
     // by more than 2^kLazyLog2; until then P may reach 2^kLazyLog2 instead of 1, which fp32 accumulators and the
@@ -251,7 +266,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const bool raise = LAZY ? (mloc * c > m_run * c + kLazyLog2) : (mloc > m_run);
     if (__builtin_amdgcn_ballot_w64(raise) != 0) {
       const float m_new = fmaxf(m_run, mloc);          // finite from the first tile on: key 0 is never masked
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      const float alpha = (BIAS && m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -259,7 +274,8 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
     }
-    const float mc = m_run * c;
+    // a bias may mask every key seen so far (-inf, e.g. left padding): the reference then stays 0 until a key counts
+    const float mc = (BIAS && m_run == -INFINITY) ? 0.0f : m_run * c;
     float psum = 0.0f;
     vec8 pf[4];
     // dropout: 32-bit index of this lane's query row at key 0 of the tile (flash_attention_triton.py:125,217)
@@ -916,14 +932,14 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
   return launch_status();
 }
 
-template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false>
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false>
 static int launch_one(const AttnParams& p, hipStream_t stream) {
   const size_t lds = 4 * (size_t)kBN * D * 2;
   const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
-  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP><<<grid, kWaves * 64, lds, stream>>>(p);
+  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS><<<grid, kWaves * 64, lds, stream>>>(p);
   return launch_status();
 }
 
@@ -931,7 +947,11 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 // WRONG results (bit 1: keep re-using the first tiles instead of copying new ones; bit 2: no exponentials).
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
-  // dropout runs on the 128-row kernel
+  // dropout and bias run on the 128-row kernel
+  if (p.bias.ptr != nullptr) {
+    if (dropout) return causal ? launch_one<T, D, true, true, 0, true, true>(p, stream) : launch_one<T, D, false, true, 0, true, true>(p, stream);
+    return causal ? launch_one<T, D, true, true, 0, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, true>(p, stream);
+  }
   if (dropout) return causal ? launch_one<T, D, true, true, 0, true>(p, stream) : launch_one<T, D, false, true, 0, true>(p, stream);
   // default: the wide kernel (eight waves x 32 rows) for head_dim 128, the 128-row kernel for head_dim 64
   // (the wide kernel addresses a head's keys with 32-bit byte offsets)
@@ -987,7 +1007,7 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
                          int B, int H, int Sq, int Sk, int D,
                          const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
                          float softmax_scale, int causal, int dtype, float dropout_p, uint32_t seed, uint64_t rng_offset,
-                         void* stream) {
+                         const void* bias, const int64_t* bias_strides, int bias_dtype, void* stream) {
   if (!q || !k || !v || !o || !qs || !ks || !vs || !os) return FO_ERR_NULL_POINTER;
   if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
   if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
@@ -1008,6 +1028,12 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   if (lse && ((uintptr_t)lse & 3u)) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;   // also rejects NaN
   if (!(dropout_p >= 0.0f) || dropout_p >= 1.0f) return FO_ERR_BAD_SHAPE;
+  if (bias) {
+    if (!bias_strides) return FO_ERR_NULL_POINTER;
+    if (bias_dtype != FO_DTYPE_F32 && bias_dtype != dtype) return FO_ERR_BAD_DTYPE;
+    if (bias_strides[0] < 0 || bias_strides[1] < 0 || bias_strides[2] < 0) return FO_ERR_BAD_STRIDE;
+    if ((uintptr_t)bias & (bias_dtype == FO_DTYPE_F32 ? 3u : 1u)) return FO_ERR_MISALIGNED;
+  }
 
   AttnParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
@@ -1017,6 +1043,9 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   p.n_qblk = (int)n_qblk;
   const bool drop = dropout_p > 0.0f;
   p.drop = make_dropout(dropout_p, seed, rng_offset);
+  p.bias.ptr = bias;
+  for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
+  p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == FO_DTYPE_BF16) return D == 128 ? launch<__bf16, 128>(p, causal != 0, drop, s) : launch<__bf16, 64>(p, causal != 0, drop, s);
   return D == 128 ? launch<_Float16, 128>(p, causal != 0, drop, s) : launch<_Float16, 64>(p, causal != 0, drop, s);
@@ -1026,7 +1055,7 @@ extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o,
                            int B, int H, int Sq, int Sk, int D,
                            const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
                            float softmax_scale, int causal, int dtype, void* stream) {
-  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, 0.0f, 0u, 0ull, stream);
+  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, 0.0f, 0u, 0ull, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int fo_attn_fwd_dropout(const void* q, const void* k, const void* v, void* o, float* lse,
@@ -1034,5 +1063,14 @@ extern "C" int fo_attn_fwd_dropout(const void* q, const void* k, const void* v, 
                                    const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
                                    float softmax_scale, int causal, int dtype, float dropout_p, uint32_t seed, uint64_t rng_offset,
                                    void* stream) {
-  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, dropout_p, seed, rng_offset, stream);
+  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, dropout_p, seed, rng_offset, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int fo_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, float* lse,
+                              int B, int H, int Sq, int Sk, int D,
+                              const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                              float softmax_scale, int causal, int dtype, const fo_attn_extras* extras, void* stream) {
+  if (!extras) return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, 0.0f, 0u, 0ull, nullptr, nullptr, 0, stream);
+  return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, extras->dropout_p,
+                       extras->dropout_seed, extras->dropout_offset, extras->bias, extras->bias_strides, extras->bias_dtype, stream);
 }

@@ -10,7 +10,7 @@ the reference leaves unimplemented (flash_attention.py:40-45) is implemented too
 
 Keyword-only extras that the reference's README promises or its Triton surface already has
 (flash_attention/README.md:34-38, flash_attention_triton.py:722-731): ``causal``, ``softmax_scale``, ``return_lse``.
-``flash_attn`` is the [B, S, H, D] surface of ``flash_attn_triton`` without bias and dropout.
+``flash_attn`` is the [B, S, H, D] surface of ``flash_attn_triton``, with its additive bias and its dropout.
 """
 from __future__ import annotations
 
@@ -46,6 +46,38 @@ def _check_inputs(q: Tensor, k: Tensor, v: Tensor) -> None:
 Dropout = Tuple[float, int, int]   # (dropout_p, seed, generator offset)
 
 
+class _AttnExtras(ctypes.Structure):    # fo_attn_extras
+    _fields_ = [("bias", ctypes.c_void_p), ("bias_strides", ctypes.c_int64 * 3), ("bias_dtype", ctypes.c_int),
+                ("dropout_p", ctypes.c_float), ("dropout_seed", ctypes.c_uint32), ("dropout_offset", ctypes.c_uint64)]
+
+
+def _expand_bias(bias: Tensor, q: Tensor, B: int, H: int, Sq: int, Sk: int) -> Tensor:
+    """The reference's checks and broadcast of the bias (flash_attention_triton.py:752-768): 4-dimensional, the dtype
+    of q or fp32, last two dimensions (1, Sk) or (Sq, Sk), expanded (strides of 0) over batch, heads and queries."""
+    if bias.dtype not in (q.dtype, torch.float32):
+        raise RuntimeError("bias must have the dtype of q or float32")
+    if not bias.is_cuda or bias.device != q.device:
+        raise RuntimeError("bias must be on the device of q")
+    if bias.dim() != 4:
+        raise RuntimeError("bias must be 4-dimensional")
+    if bias.stride(-1) != 1:
+        bias = bias.contiguous()
+    if tuple(bias.shape[2:]) not in ((1, Sk), (Sq, Sk)):
+        raise RuntimeError("Last 2 dimensions of bias must be (1, seqlen_k) or (seqlen_q, seqlen_k)")
+    return bias.expand(B, H, Sq, Sk)
+
+
+def _extras(bias: Optional[Tensor], dropout: Optional[Dropout]) -> _AttnExtras:
+    ex = _AttnExtras()
+    if bias is not None:
+        ex.bias = bias.data_ptr()
+        ex.bias_strides = _I64x3(bias.stride(0), bias.stride(1), bias.stride(2))
+        ex.bias_dtype = _lib.FO_DTYPE_F32 if bias.dtype == torch.float32 else _DTYPE_CODE[bias.dtype]
+    if dropout is not None:
+        ex.dropout_p, ex.dropout_seed, ex.dropout_offset = float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64)
+    return ex
+
+
 def next_dropout_state(n_elements: int) -> Tuple[int, int]:
     """(seed, offset) for a dropout mask over ``n_elements`` attention probabilities, taken from torch's generator of the
     current device, whose offset is advanced past them: what increment_philox_state does in the reference
@@ -60,10 +92,11 @@ def next_dropout_state(n_elements: int) -> Tuple[int, int]:
 
 def attn_fwd_strided(
     q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int], causal: bool, softmax_scale: Optional[float],
-    dropout: Optional[Dropout] = None,
+    dropout: Optional[Dropout] = None, bias: Optional[Tensor] = None,
 ) -> Tuple[Tensor, Tensor]:
-    """Launches fo_attn_fwd (fo_attn_fwd_dropout when ``dropout`` is given). ``dims`` = positions of (batch, head,
-    sequence, head_dim) in the tensors' shapes. Returns (O with q's shape, dtype and layout; LSE fp32 [B, H, Sq])."""
+    """Launches fo_attn_fwd (fo_attn_fwd_dropout when ``dropout`` is given, fo_attn_fwd_ex when ``bias`` is). ``dims`` =
+    positions of (batch, head, sequence, head_dim) in the tensors' shapes; ``bias`` is [B|1, H|1, Sq|1, Sk] whatever
+    ``dims`` says. Returns (O with q's shape, dtype and layout; LSE fp32 [B, H, Sq])."""
     _check_inputs(q, k, v)
     ib, ih, is_, id_ = dims
     B, H, Sq, D = q.shape[ib], q.shape[ih], q.shape[is_], q.shape[id_]
@@ -81,7 +114,7 @@ def attn_fwd_strided(
         # columns of V only produce output columns that are dropped; the scale stays that of the true head_dim.
         Dp = 64 if D < 64 else 128
         pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
-        o_p, lse = attn_fwd_strided(pad(q), pad(k), pad(v), dims, causal, scale, dropout)
+        o_p, lse = attn_fwd_strided(pad(q), pad(k), pad(v), dims, causal, scale, dropout, bias)
         o = torch.empty_like(q)
         o.copy_(o_p.narrow(id_, 0, D))
         return o, lse
@@ -90,12 +123,16 @@ def attn_fwd_strided(
         o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
     strides = lambda t: _I64x3(t.stride(ib), t.stride(ih), t.stride(is_))
+    if bias is not None:
+        bias = _expand_bias(bias, q, B, H, Sq, Sk)
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
                 B, H, Sq, Sk, D, strides(q), strides(k), strides(v), strides(o),
                 scale, int(bool(causal)), _DTYPE_CODE[q.dtype])
-        if dropout is None or dropout[0] == 0.0:
+        if bias is not None:
+            status = _lib.load().fo_attn_fwd_ex(*args, ctypes.byref(_extras(bias, dropout)), stream)
+        elif dropout is None or dropout[0] == 0.0:
             status = _lib.load().fo_attn_fwd(*args, stream)
         else:
             status = _lib.load().fo_attn_fwd_dropout(*args, float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64), stream)
@@ -105,7 +142,7 @@ def attn_fwd_strided(
 
 def attn_bwd_strided(
     q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor, d_o: Tensor, dims: Tuple[int, int, int, int], causal: bool,
-    softmax_scale: Optional[float], dropout: Optional[Dropout] = None,
+    softmax_scale: Optional[float], dropout: Optional[Dropout] = None, bias: Optional[Tensor] = None,
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """Launches fo_attn_bwd. Returns (dQ, dK, dV) with the shapes and dtypes of q, k, v (dense; a K/V whose heads are
     an expanded view gets a full-size gradient, which autograd then reduces)."""
@@ -120,7 +157,7 @@ def attn_bwd_strided(
         # same zero padding as the forward; O's padded columns are zero, so delta and the padded gradient columns are too
         Dp = 64 if D < 64 else 128
         pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
-        dq, dk, dv = attn_bwd_strided(pad(q), pad(k), pad(v), pad(o), lse, pad(d_o), dims, causal, scale, dropout)
+        dq, dk, dv = attn_bwd_strided(pad(q), pad(k), pad(v), pad(o), lse, pad(d_o), dims, causal, scale, dropout, bias)
         return tuple(t.narrow(id_, 0, D).contiguous() for t in (dq, dk, dv))
     if d_o.stride(-1) != 1 or any(s % 8 for s in d_o.stride()[:-1]):
         d_o = d_o.contiguous()
@@ -131,6 +168,8 @@ def attn_bwd_strided(
     dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
     delta = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    if bias is not None:
+        bias = _expand_bias(bias, q, B, H, Sq, Sk)
     tensors = (q, k, v, o, d_o, dq, dk, dv)
     arrays = [_I64x3(t.stride(ib), t.stride(ih), t.stride(is_)) for t in tensors]
     ptrs = (ctypes.POINTER(ctypes.c_int64) * 8)(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in arrays])
@@ -138,7 +177,9 @@ def attn_bwd_strided(
         stream = torch.cuda.current_stream(q.device).cuda_stream
         args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_o.data_ptr(), lse.data_ptr(), delta.data_ptr(),
                 dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, Sq, Sk, D, ptrs, scale, int(bool(causal)), _DTYPE_CODE[q.dtype])
-        if dropout is None or dropout[0] == 0.0:
+        if bias is not None:
+            status = _lib.load().fo_attn_bwd_ex(*args, ctypes.byref(_extras(bias, dropout)), stream)
+        elif dropout is None or dropout[0] == 0.0:
             status = _lib.load().fo_attn_bwd(*args, stream)
         else:
             status = _lib.load().fo_attn_bwd_dropout(*args, float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64), stream)
@@ -180,9 +221,9 @@ class _FlashAttnBSHD(Function):
 
     @staticmethod
     def forward(ctx, q: Tensor, k: Tensor, v: Tensor, causal: bool, softmax_scale: Optional[float], return_lse: bool,
-                dropout: Optional[Dropout]):
-        o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale, dropout)
-        ctx.save_for_backward(q, k, v, o, lse)
+                dropout: Optional[Dropout], bias: Optional[Tensor] = None):
+        o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale, dropout, bias)
+        ctx.save_for_backward(q, k, v, o, lse, bias)
         ctx.causal = causal
         ctx.softmax_scale = softmax_scale
         ctx.dropout = dropout
@@ -193,9 +234,11 @@ class _FlashAttnBSHD(Function):
 
     @staticmethod
     def backward(ctx, dO: Tensor, *unused):
-        q, k, v, o, lse = ctx.saved_tensors
-        dq, dk, dv = attn_bwd_strided(q, k, v, o, lse, dO, (0, 2, 1, 3), ctx.causal, ctx.softmax_scale, ctx.dropout)
-        return dq, dk, dv, None, None, None, None
+        q, k, v, o, lse, bias = ctx.saved_tensors
+        if bias is not None and ctx.needs_input_grad[7]:
+            raise RuntimeError("FlashAttention does not support bias gradient yet")   # flash_attention_triton.py:854
+        dq, dk, dv = attn_bwd_strided(q, k, v, o, lse, dO, (0, 2, 1, 3), ctx.causal, ctx.softmax_scale, ctx.dropout, bias)
+        return dq, dk, dv, None, None, None, None, None
 
 
 def _dropout_arg(dropout_p: float, dropout_state: Optional[Tuple[int, int]], n_elements: int) -> Optional[Dropout]:
@@ -236,8 +279,8 @@ def flash_attn(
     softmax_scale: Optional[float] = None, return_lse: bool = False, dropout_state: Optional[Tuple[int, int]] = None,
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """The [batch, seqlen, nheads, headdim] surface of flash_attn_triton (flash_attention_triton.py:722-737,961),
-    differentiable, with dropout. Bias is not implemented and raises."""
-    if bias is not None:
-        raise RuntimeError("attention bias is not implemented")
+    differentiable in q, k and v, with dropout and with an additive bias on the scaled scores: [B|1, H|1, 1, seqlen_k]
+    or [B|1, H|1, seqlen_q, seqlen_k], the dtype of q or fp32 (:752-768). A bias that requires grad makes the backward
+    raise, as in the reference (:854)."""
     drop = _dropout_arg(dropout_p, dropout_state, q.shape[0] * q.shape[2] * q.shape[1] * k.shape[1])
-    return _FlashAttnBSHD.apply(q, k, v, causal, softmax_scale, return_lse, drop)
+    return _FlashAttnBSHD.apply(q, k, v, causal, softmax_scale, return_lse, drop, bias)

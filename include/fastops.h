@@ -117,6 +117,30 @@ int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, const void*
                         const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
                         float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream);
 
+/* Additive bias on the scaled scores, optionally together with dropout: scores = scale * Q K^T + bias
+ * (flash_attention_triton.py:176-198,752-770; attention_ref.py:50-51). The reference's "vector" bias [.,.,1,Sk] and
+ * "matrix" bias [.,.,Sq,Sk], broadcast over batch and heads, are all expressed by strides: element (b, h, q, key) is
+ * read at bias + b*bias_strides[0] + h*bias_strides[1] + q*bias_strides[2] + key, a stride of 0 broadcasting that
+ * dimension. bias_dtype is FO_DTYPE_F32 or the dtype of q. No gradient is computed for the bias (nor does the reference).
+ * extras == NULL, or bias == NULL and dropout_p == 0, is exactly fo_attn_fwd / fo_attn_bwd. */
+typedef struct fo_attn_extras {
+  const void* bias;          /* NULL = no bias */
+  int64_t bias_strides[3];   /* element strides: batch, head, query */
+  int bias_dtype;
+  float dropout_p;           /* 0 = no dropout */
+  uint32_t dropout_seed;
+  uint64_t dropout_offset;
+} fo_attn_extras;
+int fo_attn_fwd_ex(const void* q, const void* k, const void* v, void* o, float* lse,
+                   int B, int H, int Sq, int Sk, int D,
+                   const int64_t* q_strides_host, const int64_t* k_strides_host,
+                   const int64_t* v_strides_host, const int64_t* o_strides_host,
+                   float softmax_scale, int causal, int dtype, const fo_attn_extras* extras_host, void* stream);
+int fo_attn_bwd_ex(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                   float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                   const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
+                   const fo_attn_extras* extras_host, void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------------
  * Fused Lion step: fp32 parameters, fp32 gradients, bf16 momentum, one pass.
  * Per element, in this order and with these rounding points (lion_optimizer_ref.py:51,64,65,67):

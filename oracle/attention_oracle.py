@@ -53,8 +53,11 @@ def attention_fwd_oracle(
     softmax_scale: Optional[float] = None,
     q_chunk: int = 1024,
     dropout: Optional[Tuple[float, int, int]] = None,
+    bias: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """fp32 softmax(scale * Q K^T + mask) V and its logsumexp. Returns (O fp32 [B,H,M,D], LSE fp32 [B,H,M]).
+    """fp32 softmax(scale * Q K^T + bias + mask) V and its logsumexp. Returns (O fp32 [B,H,M,D], LSE fp32 [B,H,M]).
+    ``bias`` broadcasts to [B,H,M,N] and is added to the scaled scores in fp32 (attention_ref.py:50-51,
+    flash_attention_triton.py:176-198); the logsumexp includes it.
 
     Works one (batch, head) slice and ``q_chunk`` query rows at a time so that S = 8192 does not materialise
     the full [B,H,M,N] score tensor (attention_ref.py does; same arithmetic per row).
@@ -67,6 +70,7 @@ def attention_fwd_oracle(
     out = torch.empty(B, H, M, D, dtype=torch.float32)
     lse = torch.empty(B, H, M, dtype=torch.float32)
     keep = None
+    bias_f = None if bias is None else bias.float().cpu().expand(B, H, M, N)
     if dropout is not None and dropout[0] > 0.0:
         # dropout of the probabilities after the row sums are taken (flash_attention_triton.py:203,216-219): LSE is that
         # of the undropped scores, kept probabilities are scaled by 1 / (1 - p) computed in fp32
@@ -78,6 +82,8 @@ def attention_fwd_oracle(
             for m0 in range(0, M, q_chunk):
                 m1 = min(M, m0 + q_chunk)
                 scores = (qf[b, h, m0:m1] * scale) @ kt                      # attention_ref.py:46-47
+                if bias_f is not None:
+                    scores = scores + bias_f[b, h, m0:m1]                     # attention_ref.py:50-51
                 if causal:
                     rows = torch.arange(m0, m1).unsqueeze(1)
                     cols = torch.arange(N).unsqueeze(0)
@@ -99,6 +105,7 @@ def attention_bwd_oracle(
     softmax_scale: Optional[float] = None,
     dtype: torch.dtype = torch.float32,
     dropout: Optional[Tuple[float, int, int]] = None,
+    bias: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of sum(O * dO) with respect to Q, K, V, in closed form, one (batch, head) at a time:
 
@@ -108,7 +115,8 @@ def attention_bwd_oracle(
     which is what the reference's backward computes tile by tile (flash_attention_triton.py:273-315 delta pre-pass,
     :497-578 per-tile dv / dp / ds / dk / dq) and what autograd gives for attention_ref.py:41-67. ``dtype`` is the
     arithmetic type (fp32 for the oracle proper, float64 to pin it). With dropout (mask Z = keep / (1 - p), :524-532,
-    :551,:599): O = (P * Z) V, dV = (P * Z)^T dO, dP = (dO V^T) * Z, the rest unchanged.
+    :551,:599): O = (P * Z) V, dV = (P * Z)^T dO, dP = (dO V^T) * Z, the rest unchanged. A ``bias`` (broadcast to
+    [B,H,M,N]) is added to the scaled scores before the softmax (:497-509) and gets no gradient.
     Returns (dQ, dK, dV) in ``dtype`` on the CPU.
     Pinned by tests/test_oracle_attention.py against torch.autograd on the forward expression in float64."""
     B, H, M, D = q.shape
@@ -117,12 +125,15 @@ def attention_bwd_oracle(
     qf, kf, vf, gf = (t.to(dtype).cpu() for t in (q, k, v, d_o))
     dq, dk, dv = torch.zeros_like(qf), torch.zeros_like(kf), torch.zeros_like(vf)
     z = None
+    bias_f = None if bias is None else bias.to(dtype).cpu().expand(B, H, M, N)
     if dropout is not None and dropout[0] > 0.0:
         keep = torch.from_numpy(dropout_keep_mask(dropout[0], dropout[1], dropout[2], B, H, M, N))
         z = keep.to(dtype) * float(np.float32(1.0) / (np.float32(1.0) - np.float32(dropout[0])))
     for b in range(B):
         for h in range(H):
             s = (qf[b, h] * scale) @ kf[b, h].t()
+            if bias_f is not None:
+                s = s + bias_f[b, h]
             if causal:
                 rows = torch.arange(M).unsqueeze(1)
                 cols = torch.arange(N).unsqueeze(0)

@@ -1,0 +1,146 @@
+"""Additive attention bias (flash_attention_triton.py:176-198,497-509,752-768; attention_ref.py:50-51): forward and
+backward parity with the oracle for the bias shapes the reference tests (tests/test_flash_attention_triton.py:36,
+74-82: "1h1k", "1hqk", "b11k", "b1qk"), fp32 and half-precision bias, with multi-query K/V and with dropout."""
+import math
+
+import pytest
+import torch
+
+from fast_ops.flash_attention.flash_attention import flash_attn
+from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided, attn_fwd_strided
+from oracle.attention_oracle import attention_bwd_oracle, attention_fwd_oracle, dropout_keep_mask
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+O_ATOL, O_RTOL, LSE_ATOL = 2e-2, 1e-2, 1e-3
+
+
+def _bias(kind, B, H, Sq, Sk, dtype, g):
+    shape = {"1h1k": (1, H, 1, Sk), "1hqk": (1, H, Sq, Sk), "b11k": (B, 1, 1, Sk), "b1qk": (B, 1, Sq, Sk), "bhqk": (B, H, Sq, Sk)}[kind]
+    return torch.randn(shape, generator=g).to(dtype)
+
+
+def _bshd(t):
+    return t.transpose(1, 2)    # [B,H,S,D] -> the [B,S,H,D] view flash_attn takes
+
+
+def _check(o, lse, grads, o_ref, lse_ref, grads_ref):
+    err = (o.detach().float().cpu() - o_ref).abs()
+    assert float((err - (O_ATOL + O_RTOL * o_ref.abs())).max()) <= 0, f"O: max abs err {float(err.max()):.3e}"
+    assert float((lse.cpu() - lse_ref).abs().max()) <= LSE_ATOL
+    for name, a, r in zip(("dQ", "dK", "dV"), grads, grads_ref):
+        e = (a.float().cpu() - r).abs().max().item()
+        assert e <= 2e-2 * max(1.0, r.abs().max().item()), f"{name}: error {e:.3e} vs magnitude {r.abs().max().item():.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["1h1k", "1hqk", "b11k", "b1qk", "bhqk"])
+@pytest.mark.parametrize("D", [64, 128])
+def test_bias_shapes_of_the_reference(D, kind, causal, dtype):
+    B, H, Sq, Sk = 2, 3, 200, 331      # ragged: both lengths off the tile sizes
+    g = torch.Generator().manual_seed(D + len(kind))
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk, Sq))
+    bias = _bias(kind, B, H, Sq, Sk, torch.float32, g) * 2.0
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, bias=bias)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal, bias=bias)
+    qd, kd, vd = (_bshd(t.to(DEV)).requires_grad_(True) for t in (q, k, v))
+    o, lse = flash_attn(qd, kd, vd, bias=bias.to(DEV), causal=causal, return_lse=True)
+    got = torch.autograd.grad(o, (qd, kd, vd), _bshd(go.to(DEV)))
+    torch.cuda.synchronize()
+    _check(_bshd(o), lse, [_bshd(t) for t in got], o_ref, lse_ref, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("kind", ["1h1k", "b1qk"])
+def test_bias_in_the_operand_dtype(kind, dtype):
+    # flash_attention_triton.py:755: bias.dtype in [q.dtype, torch.float]
+    B, H, Sq, Sk, D = 2, 2, 130, 257, 128
+    g = torch.Generator().manual_seed(3)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk, Sq))
+    bias = _bias(kind, B, H, Sq, Sk, dtype, g)
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=True, bias=bias)
+    ref = attention_bwd_oracle(q, k, v, go, causal=True, bias=bias)
+    qd, kd, vd = (_bshd(t.to(DEV)).requires_grad_(True) for t in (q, k, v))
+    o, lse = flash_attn(qd, kd, vd, bias=bias.to(DEV), causal=True, return_lse=True)
+    got = torch.autograd.grad(o, (qd, kd, vd), _bshd(go.to(DEV)))
+    _check(_bshd(o), lse, [_bshd(t) for t in got], o_ref, lse_ref, ref)
+    other = torch.float16 if dtype == torch.bfloat16 else torch.bfloat16
+    with pytest.raises(RuntimeError, match="dtype"):
+        flash_attn(qd, kd, vd, bias=bias.to(DEV).to(other))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_bias_with_dropout_and_multi_query(causal):
+    # the reference's test crosses bias with dropout and with K/V heads that are an expanded view (:38-39,66-72)
+    B, H, Sq, Sk, D, dtype = 2, 4, 150, 200, 64, torch.bfloat16
+    p, seed = 0.45, 4242
+    off = next(o for o in range(0, 1 << 32, (1 << 20) + 12345) if 0.25 < dropout_keep_mask(p, seed, o, B, H, Sq, Sk).mean() < 0.75)
+    g = torch.Generator().manual_seed(9)
+    q, go = (torch.randn(B, H, Sq, D, generator=g).to(dtype) for _ in range(2))
+    k1, v1 = (torch.randn(B, 1, Sk, D, generator=g).to(dtype) for _ in range(2))
+    bias = _bias("1hqk", B, H, Sq, Sk, torch.float32, g)
+    k, v = k1.expand(B, H, Sk, D), v1.expand(B, H, Sk, D)
+    drop = (p, seed, off)
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, dropout=drop, bias=bias)
+    dq_r, dk_r, dv_r = attention_bwd_oracle(q, k, v, go, causal=causal, dropout=drop, bias=bias)
+    qd = _bshd(q.to(DEV)).requires_grad_(True)
+    k1d, v1d = (t.to(DEV).requires_grad_(True) for t in (k1, v1))
+    kd, vd = (_bshd(t.expand(B, H, Sk, D)) for t in (k1d, v1d))
+    o, lse = flash_attn(qd, kd, vd, bias=bias.to(DEV), causal=causal, dropout_p=p, return_lse=True, dropout_state=(seed, off))
+    dq, dk1, dv1 = torch.autograd.grad(o, (qd, k1d, v1d), _bshd(go.to(DEV)))
+    _check(_bshd(o), lse, [_bshd(dq), dk1, dv1], o_ref, lse_ref, [dq_r, dk_r.sum(1, keepdim=True), dv_r.sum(1, keepdim=True)])
+
+
+def test_bias_as_key_padding_mask():
+    # -inf on padded keys, including the whole first tile of keys (left padding): equals attention over the kept keys.
+    # (A bias of -inf on every key of a row gives NaN in attention_ref.py:59 as well; the reference's mask_all cases
+    # compare NaN with NaN and assert nothing, tests/test_flash_attention_triton.py:86-87,131-139.)
+    B, H, S, D, dtype = 2, 2, 300, 128, torch.float16
+    g = torch.Generator().manual_seed(21)
+    q, k, v, go = (torch.randn(B, H, S, D, generator=g).to(dtype) for _ in range(4))
+    left, right = 70, 13
+    bias = torch.zeros(B, 1, 1, S)
+    bias[..., :left] = float("-inf")
+    bias[..., S - right:] = float("-inf")
+    o_ref, lse_ref = attention_fwd_oracle(q, k[:, :, left:S - right], v[:, :, left:S - right])
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o, lse = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), False, None, None, bias.to(DEV))
+    dq, dk, dv = attn_bwd_strided(qd, kd, vd, o, lse, go.to(DEV), (0, 1, 2, 3), False, None, None, bias.to(DEV))
+    dq_r, dk_r, dv_r = attention_bwd_oracle(q, k[:, :, left:S - right], v[:, :, left:S - right], go)
+    assert torch.isfinite(o.float()).all()
+    _check(o, lse, [dq, dk[:, :, left:S - right], dv[:, :, left:S - right]], o_ref, lse_ref, [dq_r, dk_r, dv_r])
+    assert float(dk[:, :, :left].abs().max()) == 0.0 and float(dv[:, :, S - right:].abs().max()) == 0.0
+
+
+def test_bias_odd_head_dim_and_large_magnitude():
+    # head_dim 40 runs on padded copies; a bias much larger than the scores decides the softmax alone
+    B, H, Sq, Sk, D, dtype = 1, 2, 100, 190, 40, torch.bfloat16
+    g = torch.Generator().manual_seed(2)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk, Sq))
+    bias = torch.randn(1, 1, Sq, Sk, generator=g) * 30.0
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=False, bias=bias)
+    ref = attention_bwd_oracle(q, k, v, go, bias=bias)
+    qd, kd, vd = (_bshd(t.to(DEV)).requires_grad_(True) for t in (q, k, v))
+    o, lse = flash_attn(qd, kd, vd, bias=bias.to(DEV), return_lse=True)
+    got = torch.autograd.grad(o, (qd, kd, vd), _bshd(go.to(DEV)))
+    _check(_bshd(o), lse, [_bshd(t) for t in got], o_ref, lse_ref, ref)
+
+
+def test_bias_rejections():
+    q = torch.randn(1, 64, 2, 64, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="Last 2 dimensions"):          # flash_attention_triton.py:764-767
+        flash_attn(q, q, q, bias=torch.zeros(1, 2, 3, 64, device=DEV))
+    with pytest.raises(RuntimeError, match="4-dimensional"):
+        flash_attn(q, q, q, bias=torch.zeros(64, 64, device=DEV))
+    # a bias that wants a gradient: the backward refuses, as the reference's does (:854)
+    qg = q.clone().requires_grad_(True)
+    bias = torch.zeros(1, 2, 64, 64, device=DEV, requires_grad=True)
+    out = flash_attn(qg, q, q, bias=bias)
+    with pytest.raises(RuntimeError, match="bias gradient"):
+        out.sum().backward()
+    # non-contiguous last dimension is made contiguous (:758-759)
+    b2 = torch.randn(1, 2, 64, 128, device=DEV)[..., ::2]
+    a = flash_attn(q, q, q, bias=b2)
+    b = flash_attn(q, q, q, bias=b2.contiguous())
+    assert torch.equal(a, b)

@@ -214,3 +214,57 @@ def test_backward_with_dropout_equals_autograd(causal):
     assert torch.allclose(o32.double(), o.detach(), rtol=1e-4, atol=1e-5)
     # LSE is that of the undropped scores
     assert torch.allclose(lse32.double(), torch.logsumexp(s.detach(), dim=-1), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["vector", "matrix"])
+def test_bias_against_library_and_invariants(causal, kind):
+    # (1) the library's additive float mask is the same thing as the reference's bias (attention_ref.py:50-51)
+    B, H, M, N, D = 2, 3, 19, 19, 16
+    q, k, v = _qkv(B, H, M, N, D, seed=11)
+    g = torch.Generator().manual_seed(12)
+    bias = torch.randn(B, H, 1 if kind == "vector" else M, N, generator=g) * 2.0
+    o, lse = attention_fwd_oracle(q, k, v, causal=causal, bias=bias)
+    mask = bias.expand(B, H, M, N).clone()
+    if causal:
+        mask = mask.masked_fill(torch.ones(M, N, dtype=torch.bool).triu(1), float("-inf"))
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+    assert torch.allclose(o, ref, atol=1e-5, rtol=1e-5)
+    s = (q @ k.transpose(-1, -2)) / math.sqrt(D) + mask
+    assert torch.allclose(lse, torch.logsumexp(s, -1), atol=1e-5, rtol=1e-6)
+    # (2) a bias constant along the keys leaves O alone and shifts the logsumexp by that constant
+    o0, lse0 = attention_fwd_oracle(q, k, v, causal=causal)
+    const = torch.randn(B, H, M, 1, generator=g).expand(B, H, M, N)
+    o1, lse1 = attention_fwd_oracle(q, k, v, causal=causal, bias=const)
+    assert torch.allclose(o1, o0, atol=1e-5, rtol=1e-5)
+    assert torch.allclose(lse1, lse0 + const[..., 0], atol=1e-5, rtol=1e-6)
+    # (3) a bias of -inf on the last keys is attention over the remaining keys; broadcast over batch and heads
+    cut = torch.zeros(1, 1, 1, N)
+    cut[..., N - 4:] = float("-inf")
+    o2, lse2 = attention_fwd_oracle(q, k, v, causal=causal, bias=cut)
+    o3, lse3 = attention_fwd_oracle(q, k[:, :, :N - 4], v[:, :, :N - 4], causal=causal)
+    assert torch.allclose(o2, o3, atol=1e-6, rtol=1e-6) and torch.allclose(lse2, lse3, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("with_dropout", [False, True])
+def test_backward_with_bias_equals_autograd(causal, with_dropout):
+    B, H, M, N, D = 2, 2, 21, 35, 8
+    drop = (0.2, 7, 123456) if with_dropout else None
+    g = torch.Generator().manual_seed(6)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g, dtype=torch.float64) for n in (M, N, N, M))
+    bias = torch.randn(1, H, M, N, generator=g, dtype=torch.float64)
+    z = 1.0
+    if drop:
+        z = torch.from_numpy(ao.dropout_keep_mask(*drop, B, H, M, N)).double() * float(np.float32(1.0) / (np.float32(1.0) - np.float32(drop[0])))
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    s = (qa / math.sqrt(D)) @ ka.transpose(-1, -2) + bias
+    if causal:
+        s = s.masked_fill(torch.arange(N)[None, :] > torch.arange(M)[:, None], float("-inf"))
+    o = (torch.softmax(s, dim=-1) * z) @ va
+    ref = torch.autograd.grad(o, (qa, ka, va), go)
+    got = ao.attention_bwd_oracle(q, k, v, go, causal=causal, dtype=torch.float64, dropout=drop, bias=bias)
+    for a, b in zip(got, ref):
+        assert torch.allclose(a, b, rtol=1e-10, atol=1e-12)
+    o32, _ = attention_fwd_oracle(q.float(), k.float(), v.float(), causal=causal, dropout=drop, bias=bias.float())
+    assert torch.allclose(o32.double(), o.detach(), rtol=1e-4, atol=1e-5)
