@@ -35,6 +35,7 @@ SIGNATURES = {
     "fo_attn_fwd": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [_I64P] * 4 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "fo_attn_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 5 + [ctypes.POINTER(_I64P), ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "fo_attn_fwd_dropout": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [_I64P] * 4 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]),
+    "fo_dropout_mask": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]),
     "fo_attn_fwd_ex": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [_I64P] * 4 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
     "fo_attn_bwd_ex": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 5 + [ctypes.POINTER(_I64P), ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
     "fo_attn_bwd_dropout": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 5 + [ctypes.POINTER(_I64P), ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]),

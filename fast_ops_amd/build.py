@@ -40,6 +40,7 @@ SOURCES = {
     # would silently leave them rolled, with their register arrays in scratch memory.
     "attn_fwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
     "attn_bwd.hip": [],
+    "dropout_mask.hip": [],
 }
 # sources whose generated assembly is checked by asm_lint: source -> regular expression of the kernel symbols to check
 # (the instantiations with a non-zero last template argument are timing experiments with wrong results by design)

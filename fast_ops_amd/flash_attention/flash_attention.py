@@ -90,6 +90,28 @@ def next_dropout_state(n_elements: int) -> Tuple[int, int]:
     return seed, offset
 
 
+def dropout_mask(
+    dropout_p: float, batch_sz: int, n_heads: int, seqlen_q: int, seqlen_k: int, device: Union[str, torch.device],
+    dropout_state: Optional[Tuple[int, int]] = None,
+) -> Tensor:
+    """The keep-mask (bool [B, H, Sq, Sk], True = kept) that the attention kernels apply for this dropout_p and state:
+    triton_dropout_mask of the reference (flash_attention_triton.py:697-717). Without ``dropout_state`` the state comes
+    from torch's generator, which is advanced exactly as an attention call of that shape advances it, so seeding, taking
+    the mask, seeding again and calling the attention gives the attention's mask (tests/test_flash_attention_triton.py:
+    93-103)."""
+    if not 0.0 <= dropout_p < 1.0:
+        raise RuntimeError(f"dropout_p must be in [0, 1), got {dropout_p}")
+    device = torch.device(device)
+    n = batch_sz * n_heads * seqlen_q * seqlen_k
+    with torch.cuda.device(device):
+        seed, offset = dropout_state if dropout_state is not None else next_dropout_state(n)
+        keep = torch.empty((batch_sz, n_heads, seqlen_q, seqlen_k), dtype=torch.uint8, device=device)
+        status = _lib.load().fo_dropout_mask(keep.data_ptr(), n, float(dropout_p), seed & 0xFFFFFFFF, offset % (1 << 64),
+                                             torch.cuda.current_stream(device).cuda_stream)
+    _lib.check(status, "fo_dropout_mask")
+    return keep.view(torch.bool)
+
+
 def attn_fwd_strided(
     q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int], causal: bool, softmax_scale: Optional[float],
     dropout: Optional[Dropout] = None, bias: Optional[Tensor] = None,

@@ -117,6 +117,11 @@ int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, const void*
                         const int64_t* const* strides_host, float softmax_scale, int causal, int dtype,
                         float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream);
 
+/* The dropout keep-mask as a tensor of its own, one byte per element of [B, H, Sq, Sk] flattened (1 = kept): what
+ * fo_attn_fwd_dropout applies for the same (dropout_p, seed, rng_offset). Replaces triton_dropout_mask's kernel
+ * (flash_attention_triton.py:669-717), which the reference's tests use to build the mask for attention_ref. */
+int fo_dropout_mask(uint8_t* keep, int64_t n_elements, float dropout_p, uint32_t seed, uint64_t rng_offset, void* stream);
+
 /* Additive bias on the scaled scores, optionally together with dropout: scores = scale * Q K^T + bias
  * (flash_attention_triton.py:176-198,752-770; attention_ref.py:50-51). The reference's "vector" bias [.,.,1,Sk] and
  * "matrix" bias [.,.,Sq,Sk], broadcast over batch and heads, are all expressed by strides: element (b, h, q, key) is

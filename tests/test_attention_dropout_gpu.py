@@ -94,3 +94,51 @@ def test_generator_state_is_consumed_like_the_reference():
     assert torch.equal(a, c)
     with pytest.raises(RuntimeError, match="dropout_p"):
         multi_head_attention(q, k, v, dropout_p=1.0)
+
+
+def test_dropout_mask_tensor_is_the_kernels_mask():
+    # triton_dropout_mask of the reference (flash_attention_triton.py:697-717): the mask as a tensor, bit for bit the
+    # oracle's, for explicit states (including a 32-bit wrap of the index) and ragged sizes that end inside a 16-byte store
+    from fast_ops.flash_attention.flash_attention_triton import flash_attn_triton, increment_philox_state, triton_dropout_mask
+    from fast_ops_amd.flash_attention.flash_attention import dropout_mask
+    for (B, H, Sq, Sk, p, seed, off) in [(2, 3, 70, 64, 0.87, 42, 5), (1, 1, 1, 1, 0.5, 7, 0), (1, 2, 33, 17, 0.3, 99, (1 << 32) - 500),
+                                         (2, 2, 128, 256, 0.17, 123, 3 << 20)]:
+        got = dropout_mask(p, B, H, Sq, Sk, DEV, dropout_state=(seed, off))
+        assert got.dtype == torch.bool and tuple(got.shape) == (B, H, Sq, Sk)
+        assert np.array_equal(got.cpu().numpy(), dropout_keep_mask(p, seed, off, B, H, Sq, Sk))
+    # the reference's test flow (tests/test_flash_attention_triton.py:93-103): seed, run the attention, seed again, take
+    # the mask: it is the mask the attention used
+    B, H, Sq, Sk, D, p = 2, 2, 96, 80, 64, 0.87
+    q, k, v, _ = (t.to(DEV).transpose(1, 2) for t in _inputs(B, H, Sq, Sk, D, torch.float16, 3))
+    torch.manual_seed(1234567)
+    increment_philox_state(_mixed_state(p, B, H, Sq, Sk, 1234567))   # to offsets where this hash mixes a small mask
+    state = torch.cuda.get_rng_state()
+    out = flash_attn_triton(q, k, v, None, False, p)
+    after = torch.cuda.get_rng_state()
+    torch.cuda.set_rng_state(state)
+    keep = triton_dropout_mask(p, B, H, Sq, Sk, device=DEV)
+    assert torch.equal(torch.cuda.get_rng_state(), after)     # both consume the generator alike
+    words = state.numpy().view(np.uint64)
+    o_ref, _ = attention_fwd_oracle(*(t.transpose(1, 2) for t in (q, k, v)), dropout=(p, int(words[-2]), int(words[-1])))
+    assert np.array_equal(keep.cpu().numpy(), dropout_keep_mask(p, int(words[-2]), int(words[-1]), B, H, Sq, Sk))
+    assert 0.2 < float(keep.float().mean()) < 0.8
+    err = (out.transpose(1, 2).float().cpu() - o_ref).abs()
+    assert float((err - (O_ATOL + O_RTOL * o_ref.abs())).max()) <= 0
+
+
+@pytest.mark.parametrize("seed", [123, 0])
+def test_dropout_statistics_like_the_reference(seed):
+    # tests/test_flash_attention_triton.py:204-236: 1000 masks from consecutive generator states; every element must be
+    # kept in a fraction of them that a binomial test against 1 - p does not reject at 1e-8. (p-values are computed per
+    # distinct count instead of per element: the same numbers without the reference's 10^6 x 10^3 table.)
+    import scipy.stats
+    from fast_ops.flash_attention.flash_attention_triton import triton_dropout_mask
+    B, H, Sq, Sk, p, n_trials = 8, 4, 128, 256, 0.17, 1000
+    torch.manual_seed(seed)
+    sums = torch.zeros(B, H, Sq, Sk, dtype=torch.int32, device=DEV)
+    for _ in range(n_trials):
+        sums += triton_dropout_mask(p, B, H, Sq, Sk, device=DEV)
+    counts = np.unique(sums.cpu().numpy())
+    pvals = {int(c): scipy.stats.binomtest(int(c), n_trials, 1.0 - p).pvalue for c in counts}
+    worst = min(pvals, key=pvals.get)
+    assert pvals[worst] > 1e-8, f"failed binomial test: kept {worst / n_trials}, expected {1 - p}, p-value {pvals[worst]}"
