@@ -21,6 +21,8 @@
 // Both recompute the scores (seven GEMMs in total instead of the five of an atomics-based single pass).
 // Tiles of 64 rows go global -> LDS with the direct-to-LDS loads, double buffered, one barrier per tile, 16-byte
 // chunks XOR-swizzled inside a row (no bank conflicts), exactly as in the 128-row forward kernel.
+#include <type_traits>
+
 #include "attn_common.hpp"
 
 namespace fo {
@@ -194,25 +196,31 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     const uint32_t drop_row = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0w + l32)) * (uint32_t)Sk + (uint32_t)key0 : 0u;
     // bias row of this lane's query (flash_attention_triton.py:497-509); keys past the end re-read the last one
     const int64_t bias_row = BIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)qrow * prm.bias.strides[2] : 0;
+    // (the factor softmax_scale of dS is applied once, to the finished accumulators; tiles that no mask touches - most -
+    // go without the comparisons)
+    auto softmax_grad = [&](auto masked) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int key_base = key0 + 32 * kb + 4 * hh;
-      int lim = key_base - Sk + 1;
-      if (CAUSAL) lim = max(lim, key_base - (q0w + l32));
+      for (int kb = 0; kb < 2; ++kb) {
+        const int key_base = key0 + 32 * kb + 4 * hh;
+        int lim = key_base - Sk + 1;
+        if (CAUSAL) lim = max(lim, key_base - (q0w + l32));
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const bool dead = lim > -((r & 3) + 8 * (r >> 2));
-        float shift = -lse2;
-        if constexpr (BIAS) shift = __builtin_fmaf(load_bias<T>(prm.bias, bias_row + min(key_base + (r & 3) + 8 * (r >> 2), Sk - 1)), kLog2e, -lse2);
-        const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, shift));
-        float dp = dpacc[kb][r];
-        if constexpr (DROP) {
-          const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2));
-          dp = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? dp * prm.drop.keep_scale : 0.0f;
+        for (int r = 0; r < 16; ++r) {
+          const bool dead = decltype(masked)::value && lim > -((r & 3) + 8 * (r >> 2));
+          float shift = -lse2;
+          if constexpr (BIAS) shift = __builtin_fmaf(load_bias<T>(prm.bias, bias_row + min(key_base + (r & 3) + 8 * (r >> 2), Sk - 1)), kLog2e, -lse2);
+          const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, shift));
+          float dp = dpacc[kb][r];
+          if constexpr (DROP) {
+            const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2));
+            dp = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? dp * prm.drop.keep_scale : 0.0f;
+          }
+          dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp - delta));
         }
-        dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp - delta) * scale);
       }
-    }
+    };
+    if (key0 + kBwdTile > Sk || (CAUSAL && key0 + kBwdTile - 1 > q0w)) softmax_grad(std::true_type{});
+    else softmax_grad(std::false_type{});
     // dQ^T += K^T dS^T : four 16-key steps x DBLK d-blocks
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -230,7 +238,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
         typedef __attribute__((ext_vector_type(4))) T vec4;
         vec4 o4;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) o4[u] = (T)acc[db][rg * 4 + u];
+        for (int u = 0; u < 4; ++u) o4[u] = (T)(acc[db][rg * 4 + u] * scale);
         *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
       }
   }
@@ -323,6 +331,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
       const uint32_t drop_base = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0t + 32 * qb + 4 * hh)) * (uint32_t)Sk + (uint32_t)key : 0u;
       // bias column of this lane's key; queries past the end re-read the last one
       const int64_t bias_col = BIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] + krow : 0;
+      auto softmax_grad = [&](auto masked) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 l4 = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * j + 4 * hh);
@@ -330,7 +339,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           const int r = 4 * j + u;
-          const bool dead = (u + 8 * j) < lim || (u + 8 * j) >= lim_end;
+          const bool dead = decltype(masked)::value && ((u + 8 * j) < lim || (u + 8 * j) >= lim_end);
           float shift = -l4[u] * kLog2e;
           if constexpr (BIAS) {
             const int qi = min(q0t + 32 * qb + 4 * hh + u + 8 * j, Sq - 1);
@@ -344,9 +353,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
             dp = keep ? dp * prm.drop.keep_scale : 0.0f;
           }
           pf[r >> 3][r & 7] = (T)pd;
-          dsf[r >> 3][r & 7] = (T)(p * (dp - d4[u]) * scale);
+          dsf[r >> 3][r & 7] = (T)(p * (dp - d4[u]));   // softmax_scale is applied to the finished dK
         }
       }
+      };
+      if (q0t + 32 * qb + 32 > Sq || (CAUSAL && k0w + 31 > q0t + 32 * qb)) softmax_grad(std::true_type{});
+      else softmax_grad(std::false_type{});
       // dV^T += dO^T P and dK^T += Q^T dS : two 16-query steps x DBLK d-blocks
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -368,7 +380,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
         typedef __attribute__((ext_vector_type(4))) T vec4;
         vec4 k4, v4;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) { k4[u] = (T)dkacc[db][rg * 4 + u]; v4[u] = (T)dvacc[db][rg * 4 + u]; }
+        for (int u = 0; u < 4; ++u) { k4[u] = (T)(dkacc[db][rg * 4 + u] * scale); v4[u] = (T)dvacc[db][rg * 4 + u]; }
         *(vec4*)(kp + 32 * db + 8 * rg + 4 * hh) = k4;
         *(vec4*)(vp + 32 * db + 8 * rg + 4 * hh) = v4;
       }
