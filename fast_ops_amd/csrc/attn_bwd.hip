@@ -45,6 +45,35 @@ struct AttnBwdParams {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// acc += A B with the accumulator pinned in AGPRs. Left to the compiler, the 128 accumulator registers of dK and dV are
+// kept elsewhere between uses and copied in and out around every MFMA (eight extra VALU instructions per MFMA). Inside
+// an asm statement the compiler's hazard recognizer does not see the MFMA, so: two wait states in front (a source may
+// have just been written by a VALU instruction, e.g. a register copy), and acc_fence() before anything but such an
+// MFMA touches an accumulator. FO_MFMA_NOPS=1 (the build's fallback when its check of the generated assembly finds a
+// hazard) uses the builtin instead.
+#ifndef FO_MFMA_NOPS
+#define FO_MFMA_NOPS 0
+#endif
+template <typename T>
+__device__ __forceinline__ void mfma_acc_agpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b) {
+#if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
+  if constexpr (std::is_same<T, __bf16>::value)
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  else
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+#else
+  acc = Ops<T>::mfma(a, b, acc);
+#endif
+}
+template <int N>
+__device__ __forceinline__ void acc_fence(f32x16 (&acc)[N]) {
+#if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
+  asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+a"(acc[i]));
+#endif
+}
+
 // ---------------------------------------------------------------------------------------------------------------------
 // delta[b, h, q] = sum_d dO * O   (flash_attention_triton.py:273-315). Eight lanes per row.
 template <typename T, int D>
@@ -387,6 +416,214 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// dK/dV without dropout and bias, as a software pipeline. The accumulators of dK and dV, the K^T and V^T fragments and
+// two blocks of scores leave room for one wave per SIMD only, and a lone wave issues in order: whatever arithmetic sits
+// between two MFMAs keeps the matrix pipe waiting unless it is laid out to run beside them. A 64-query tile is two
+// 32-query blocks and four phases of NMF MFMAs each:
+//   1: S, dP of block 0 | 2: S, dP of block 1 + softmax gradient of block 0 | 3: dV, dK of block 0 + softmax gradient of
+//   block 1 | 4: dV, dK of block 1
+// as micro-groups of one MFMA, the LDS read of the A operand needed kFragAhead groups later and, in phases 2 and 3, one
+// or two score elements, fenced so that the compiler keeps the groups apart.
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(const AttnBwdParams prm) {
+  typedef typename Ops<T>::vec8 vec8;
+  constexpr int TILE_BYTES = kBwdTile * D * 2;
+  constexpr int KSTEPS = D / 16;
+  constexpr int DBLK = D / 32;
+  constexpr int NMF = 2 * KSTEPS;           // MFMAs per phase (= 4 * DBLK)
+  constexpr int EPG = 16 / NMF;             // score elements per micro-group
+  static_assert(4 * DBLK == NMF && EPG >= 1, "phases of equal length");
+  extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q0 | Q1 | dO0 | dO1 | lse[2][64] | delta[2][64]
+  FO_LDS float* rowvals = (FO_LDS float*)(smem + 4 * TILE_BYTES);
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+  const int n_bh = prm.B * prm.H;
+  const int bh = blockIdx.x % n_bh;
+  const int kblk = blockIdx.x / n_bh;                 // key block 0 has the most queries when causal: heaviest first
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int k0 = kblk * kBwdRows, k0w = k0 + wave_s * 32;
+  const int Sq = prm.Sq, Sk = prm.Sk;
+  const T* qbase = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  const T* gbase = (const T*)prm.d_o + b * prm.dos[0] + h * prm.dos[1];
+  const int n_qt = (Sq + kBwdTile - 1) / kBwdTile;
+  const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;     // queries before the block's first key never attend it
+  const int ja = CAUSAL ? min(k0w / kBwdTile, n_qt) : 0;     // ... and this wave's keys start later still
+
+  auto issue = [&](int qt, int buf) {
+    copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
+    copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    if (wave_s < 2) {
+      const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
+      dma4_lane_ptr((wave_s == 0 ? prm.lse : (const float*)prm.delta) + at, rowvals + (2 * wave_s + buf) * kBwdTile);
+    }
+  };
+  if (qt0 < n_qt) issue(qt0, 0);
+  // hand-over j: tile j+1 has landed for everyone, nobody reads tile j any more, the copy of tile j+2 may start.
+  // Every wave runs hand-overs qt0-1 .. n_qt-2, each exactly once.
+  auto hand_over = [&](int j) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (j + 2 < n_qt) issue(j + 2, (j + 2 - qt0) & 1);
+  };
+
+  const int key = k0w + l32;
+  const int krow = min(key, Sk - 1);
+  vec8 kf[KSTEPS], vf[KSTEPS];
+  {
+    const T* kp = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1] + (int64_t)krow * prm.ks[2] + 8 * hh;
+    const T* vp = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1] + (int64_t)krow * prm.vs[2] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) { kf[ks] = *(const vec8*)(kp + 16 * ks); vf[ks] = *(const vec8*)(vp + 16 * ks); }
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(kf[ks]), "v"(vf[ks]));
+  }
+  f32x16 dkacc[DBLK], dvacc[DBLK];
+#pragma unroll
+  for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.0f; dvacc[i][r] = 0.0f; }
+  const float c = prm.scale_log2e, scale = prm.scale;
+
+  // A operand of MFMA i of a scores phase (even i: Q rows for S, odd i: dO rows for dP) / of a gradient phase (even i:
+  // dO^T for dV, odd i: Q^T for dK)
+  auto scores_frag = [&](FO_LDS const char* qtile, FO_LDS const char* gtile, int qb, int i) -> vec8 {
+    return row_frag<T, D>((i & 1) ? gtile : qtile, qb, i >> 1, l32, hh);
+  };
+  auto grads_frag = [&](FO_LDS const char* qtile, FO_LDS const char* gtile, int qb, int i) -> vec8 {
+    return col_frag<T, D>((i & 1) ? qtile : gtile, 2 * qb + i / (2 * DBLK), (i >> 1) % DBLK, lane);
+  };
+  constexpr int kFragAhead = 3;
+  vec8 fr[kFragAhead];         // A operands, fetched kFragAhead micro-groups ahead of their MFMA
+  f32x16 sacc[2], dpacc[2];
+  vec8 pf[2][2], dsf[2][2];
+
+  auto tile_body = [&](int j, auto masked) {
+    const int buf = (j - qt0) & 1;
+    const int q0t = j * kBwdTile;
+    FO_LDS const char* qtile = smem + buf * TILE_BYTES;
+    FO_LDS const char* gtile = smem + (2 + buf) * TILE_BYTES;
+    // A operand of the tile's MFMA g (phases of NMF)
+    auto frag = [&](int g) -> vec8 {
+      const int ph = g / NMF, i = g % NMF;
+      return ph < 2 ? scores_frag(qtile, gtile, ph, i) : grads_frag(qtile, gtile, ph - 2, i);
+    };
+    auto refill = [&](int g) { if (g + kFragAhead < 4 * NMF) fr[g % kFragAhead] = frag(g + kFragAhead); };
+    FO_LDS const float* lse_t = rowvals + buf * kBwdTile;
+    FO_LDS const float* del_t = rowvals + (2 + buf) * kBwdTile;
+    f32x4 lv[2], dv[2];        // LSE and delta of four query rows, fetched one vector ahead
+    // score element r of block qb: register r holds query q0t + 32*qb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2);
+    // dead iff key > query or the query is past the end
+    auto element = [&](int qb, int r) {
+      const int jv = r >> 2, u = r & 3;
+      if (u == 0 && jv + 1 < 4) {
+        lv[(jv + 1) & 1] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * (jv + 1) + 4 * hh);
+        dv[(jv + 1) & 1] = *(FO_LDS const f32x4*)(del_t + 32 * qb + 8 * (jv + 1) + 4 * hh);
+      }
+      const int koff = u + 8 * jv;
+      bool dead = false;
+      if constexpr (decltype(masked)::value) {
+        const int lim = CAUSAL ? key - (q0t + 32 * qb + 4 * hh) : 0;
+        const int lim_end = Sq - (q0t + 32 * qb + 4 * hh);
+        dead = koff < lim || koff >= lim_end;
+      }
+      const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][r], c, -lv[jv & 1][u] * kLog2e));
+      pf[qb][r >> 3][r & 7] = (T)p;
+      dsf[qb][r >> 3][r & 7] = (T)(p * (dpacc[qb][r] - dv[jv & 1][u]));   // softmax_scale is applied to the finished dK
+    };
+    auto first_rows = [&](int qb) {
+      lv[0] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 4 * hh);
+      dv[0] = *(FO_LDS const f32x4*)(del_t + 32 * qb + 4 * hh);
+    };
+    // ---- phase 1
+#pragma unroll
+    for (int i = 0; i < kFragAhead; ++i) fr[i] = frag(i);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { sacc[0][r] = 0.0f; dpacc[0][r] = 0.0f; sacc[1][r] = 0.0f; dpacc[1][r] = 0.0f; }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NMF; ++i) {
+      const int g = i;
+      if (i & 1) dpacc[0] = Ops<T>::mfma(fr[g % kFragAhead], vf[i >> 1], dpacc[0]); else sacc[0] = Ops<T>::mfma(fr[g % kFragAhead], kf[i >> 1], sacc[0]);
+      refill(g);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- phase 2
+    first_rows(0);
+#pragma unroll
+    for (int i = 0; i < NMF; ++i) {
+      const int g = NMF + i;
+      if (i & 1) dpacc[1] = Ops<T>::mfma(fr[g % kFragAhead], vf[i >> 1], dpacc[1]); else sacc[1] = Ops<T>::mfma(fr[g % kFragAhead], kf[i >> 1], sacc[1]);
+      refill(g);
+#pragma unroll
+      for (int e = 0; e < EPG; ++e) element(0, i * EPG + e);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- phase 3
+    first_rows(1);
+#pragma unroll
+    for (int i = 0; i < NMF; ++i) {
+      const int g = 2 * NMF + i;
+      const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
+      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], dsf[0][t]); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], pf[0][t]);
+      refill(g);
+#pragma unroll
+      for (int e = 0; e < EPG; ++e) element(1, i * EPG + e);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- phase 4
+#pragma unroll
+    for (int i = 0; i < NMF; ++i) {
+      const int g = 3 * NMF + i;
+      const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
+      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], dsf[1][t]); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], pf[1][t]);
+      refill(g);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  int j = qt0 - 1;
+  for (; j <= min(ja, n_qt) - 1 && j <= n_qt - 2; ++j) hand_over(j);
+  // Tiles that need the mask are a prefix (the causal diagonal) and possibly the last tile (queries past the end).
+  // One loop per kind, each with a single body: with alternatives inside one loop the compiler moves the 128
+  // accumulator registers between homes at every tile.
+  auto needs_mask = [&](int jt) { return jt * kBwdTile + kBwdTile > Sq || (CAUSAL && k0w + 31 > jt * kBwdTile); };
+  j = ja;
+  for (; j < n_qt && needs_mask(j); ++j) {
+    tile_body(j, std::true_type{});
+    if (j + 1 < n_qt) hand_over(j);
+  }
+  for (; j < n_qt && !needs_mask(j); ++j) {
+    tile_body(j, std::false_type{});
+    if (j + 1 < n_qt) hand_over(j);
+  }
+  for (; j < n_qt; ++j) {
+    tile_body(j, std::true_type{});
+    if (j + 1 < n_qt) hand_over(j);
+  }
+
+  acc_fence(dkacc);
+  acc_fence(dvacc);
+  if (key < Sk) {
+    T* kp = (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1] + (int64_t)key * prm.dks[2];
+    T* vp = (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1] + (int64_t)key * prm.dvs[2];
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        typedef __attribute__((ext_vector_type(4))) T vec4;
+        vec4 k4, v4;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { k4[u] = (T)(dkacc[db][rg * 4 + u] * scale); v4[u] = (T)dvacc[db][rg * 4 + u]; }
+        *(vec4*)(kp + 32 * db + 8 * rg + 4 * hh) = k4;
+        *(vec4*)(vp + 32 * db + 8 * rg + 4 * hh) = v4;
+      }
+  }
+}
+
 template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
 static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
@@ -401,10 +638,14 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
   static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
-  if (a1 != hipSuccess || a2 != hipSuccess) return FO_ERR_LAUNCH;
+  static const hipError_t a3 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+  if (a1 != hipSuccess || a2 != hipSuccess || a3 != hipSuccess) return FO_ERR_LAUNCH;
   attn_bwd_delta_kernel<T, D><<<(unsigned)g_delta, 256, 0, s>>>(p);
   attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
-  attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
+  // attn_bwd.variant 0 selects the plain dK/dV kernel everywhere (tests compare the two)
+  if (!DROP && !BIAS && g_attn_bwd_variant != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
+  else attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
   return launch_status();
 }
 

@@ -36,12 +36,12 @@ __device__ __forceinline__ float half_swap(float x) {
 // device pass only.)
 __device__ __forceinline__ void dma16_uniform_base(const void* base, uint32_t byte_off, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"((uint32_t)(uintptr_t)dst), "v"(byte_off), "s"(base) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(byte_off), "s"(base) : "memory", "m0");
 #endif
 }
 __device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"((uint32_t)(uintptr_t)dst), "v"(ptr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
 #endif
 }
 
@@ -88,7 +88,7 @@ __device__ __forceinline__ float load_bias(const BiasParams& bp, int64_t at) {
 // the same with 4 bytes per lane (LDS receives 256 bytes)
 __device__ __forceinline__ void dma4_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"((uint32_t)(uintptr_t)dst), "v"(ptr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
 #endif
 }
 

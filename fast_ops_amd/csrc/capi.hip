@@ -6,6 +6,7 @@
 namespace fo {
 int g_lion_variant = -1;
 int g_attn_variant = -1;
+int g_attn_bwd_variant = -1;
 }  // namespace fo
 
 extern "C" const char* fo_strerror(int status) {
@@ -30,6 +31,7 @@ extern "C" int fo_tune_set(const char* key, int value) {
   if (value < -1) return FO_ERR_UNSUPPORTED;
   if (strcmp(key, "lion.variant") == 0) { fo::g_lion_variant = value; return FO_OK; }
   if (strcmp(key, "attn.variant") == 0) { fo::g_attn_variant = value; return FO_OK; }
+  if (strcmp(key, "attn_bwd.variant") == 0) { fo::g_attn_bwd_variant = value; return FO_OK; }
   return FO_ERR_UNSUPPORTED;
 }
 
@@ -37,5 +39,6 @@ extern "C" int fo_tune_get(const char* key) {
   if (!key) return FO_ERR_NULL_POINTER;
   if (strcmp(key, "lion.variant") == 0) return fo::g_lion_variant;
   if (strcmp(key, "attn.variant") == 0) return fo::g_attn_variant;
+  if (strcmp(key, "attn_bwd.variant") == 0) return fo::g_attn_bwd_variant;
   return FO_ERR_UNSUPPORTED;
 }

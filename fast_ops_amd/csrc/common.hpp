@@ -21,6 +21,7 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 // variant selectors set through fo_tune_set (-1 = default)
 extern int g_lion_variant;
 extern int g_attn_variant;
+extern int g_attn_bwd_variant;
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? FO_OK : FO_ERR_LAUNCH; }
 

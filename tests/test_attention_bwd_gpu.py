@@ -59,18 +59,33 @@ def _run(B, H, Sq, Sk, D, dtype, causal, seed=0, scale=None):
     _check(got, ref, pt, f"B{B} H{H} Sq{Sq} Sk{Sk} D{D} {dtype} causal={causal}")
 
 
+@pytest.fixture(params=[-1, 0], ids=["dkdv-pipelined", "dkdv-plain"])
+def dkdv_variant(request):
+    """Both dK/dV kernels: the software-pipelined one (default without dropout and bias) and the plain one."""
+    from fast_ops_amd import _lib
+    _lib.tune_set("attn_bwd.variant", request.param)
+    yield request.param
+    _lib.tune_set("attn_bwd.variant", -1)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
-def test_dtype_causal_headdim_grid(dtype, causal, D):
+def test_dtype_causal_headdim_grid(dtype, causal, D, dkdv_variant):
     _run(2, 3, 256, 256, D, dtype, causal, seed=D)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_long_sequence_many_tiles_per_key_block(causal, dkdv_variant):
+    # 1024 queries = 16 tiles per key block: the steady state of the tile pipeline, and (causal) every wave's own start
+    _run(1, 2, 1024, 1024, 128, torch.bfloat16, causal, seed=11)
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 300),
                                    (1, 1, 300, 64), (2, 2, 191, 191), (1, 1, 385, 513)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
-def test_ragged_and_unequal_lengths(shape, causal, D):
+def test_ragged_and_unequal_lengths(shape, causal, D, dkdv_variant):
     # lengths that are not multiples of the 128-row blocks / 64-row tiles, Sq != Sk (causal mask top-left aligned: keys
     # beyond the last query get exactly zero gradient)
     B, H, Sq, Sk = shape
