@@ -47,10 +47,10 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 // acc += A B with the accumulator pinned in AGPRs. Left to the compiler, the 128 accumulator registers of dK and dV are
 // kept elsewhere between uses and copied in and out around every MFMA (eight extra VALU instructions per MFMA). Inside
-// an asm statement the compiler's hazard recognizer does not see the MFMA, so: two wait states in front (a source may
-// have just been written by a VALU instruction, e.g. a register copy), and acc_fence() before anything but such an
-// MFMA touches an accumulator. FO_MFMA_NOPS=1 (the build's fallback when its check of the generated assembly finds a
-// hazard) uses the builtin instead.
+// an asm statement the compiler's hazard recognizer does not see the MFMA: no source may have been written by a VALU
+// instruction (a register copy, say) in the two instructions before it, and nothing but such an MFMA may touch an
+// accumulator before acc_fence(). The build checks the generated assembly for both (fast_ops_amd/asm_lint.py) and
+// falls back to FO_MFMA_NOPS=1, the builtin, if it finds a violation.
 #ifndef FO_MFMA_NOPS
 #define FO_MFMA_NOPS 0
 #endif
@@ -58,11 +58,36 @@ template <typename T>
 __device__ __forceinline__ void mfma_acc_agpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b) {
 #if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
   if constexpr (std::is_same<T, __bf16>::value)
-    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
   else
-    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 #else
   acc = Ops<T>::mfma(a, b, acc);
+#endif
+}
+// S / dP of the pipelined dK/dV kernel: result pinned in VGPRs (the softmax gradient reads it element by element; from
+// AGPRs every read is an extra instruction). `first` starts a new sum. Readers wait with scores_fence().
+template <typename T>
+__device__ __forceinline__ void mfma_scores_vgpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b, bool first) {
+#if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
+  if constexpr (std::is_same<T, __bf16>::value) {
+    if (first) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+  } else {
+    if (first) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+  }
+#else
+  if (first) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  }
+  acc = Ops<T>::mfma(a, b, acc);
+#endif
+}
+__device__ __forceinline__ void scores_fence(f32x16& s, f32x16& dp) {
+#if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
+  asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s), "+v"(dp));
 #endif
 }
 template <int N>
@@ -435,8 +460,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   constexpr int EPG = 16 / NMF;             // score elements per micro-group
   static_assert(4 * DBLK == NMF && EPG >= 1, "phases of equal length");
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q0 | Q1 | dO0 | dO1 | lse[2][64] | delta[2][64]
-  FO_LDS float* rowvals = (FO_LDS float*)(smem + 4 * TILE_BYTES);
+  constexpr int NBUF = 3;                   // tile buffers: see hand_over()
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q[NBUF] | dO[NBUF] | lse[NBUF][64] | delta[NBUF][64]
+  FO_LDS float* rowvals = (FO_LDS float*)(smem + 2 * NBUF * TILE_BYTES);
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
@@ -455,19 +481,21 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 
   auto issue = [&](int qt, int buf) {
     copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
-    copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (NBUF + buf) * TILE_BYTES, wave_s, lane);
     if (wave_s < 2) {
       const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
-      dma4_lane_ptr((wave_s == 0 ? prm.lse : (const float*)prm.delta) + at, rowvals + (2 * wave_s + buf) * kBwdTile);
+      dma4_lane_ptr((wave_s == 0 ? prm.lse : (const float*)prm.delta) + at, rowvals + (NBUF * wave_s + buf) * kBwdTile);
     }
   };
   if (qt0 < n_qt) issue(qt0, 0);
-  // hand-over j: tile j+1 has landed for everyone, nobody reads tile j any more, the copy of tile j+2 may start.
-  // Every wave runs hand-overs qt0-1 .. n_qt-2, each exactly once.
+  // hand-over j, between phases 3 and 4 of tile j: tile j+1 (copy started one tile ago) has landed for everyone, and
+  // since everyone is past phase 3 of tile j nobody reads tile j-1 any more, whose buffer - the third one - takes the
+  // copy of tile j+2. Phase 4 still reads tile j, and already fetches the first fragments of tile j+1, so the fragment
+  // pipeline never drains. Every wave runs hand-overs qt0-1 .. n_qt-2, each exactly once.
   auto hand_over = [&](int j) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (j + 2 < n_qt) issue(j + 2, (j + 2 - qt0) & 1);
+    __builtin_amdgcn_s_barrier();
+    if (j + 2 < n_qt) issue(j + 2, (j + 2 - qt0) % NBUF);
   };
 
   const int key = k0w + l32;
@@ -488,32 +516,66 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.0f; dvacc[i][r] = 0.0f; }
   const float c = prm.scale_log2e, scale = prm.scale;
 
+  // Per-lane byte offsets of the fragment reads inside a tile, swizzle included (what row_frag / col_frag compute; the
+  // swizzle of a row does not depend on the 32-row block or 16-row step it is in). With the tile's base added once
+  // per tile every read is register + immediate: block, step and the dO tiles (NBUF tiles behind the Q tiles) are
+  // immediates.
+  constexpr int ROW = D * 2;
+  constexpr int G_OFF = NBUF * TILE_BYTES;
+  uint32_t row_off[KSTEPS], col_off[DBLK][2];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) row_off[ks] = (uint32_t)(l32 * ROW + (((2 * ks + hh) ^ swz<D>(l32)) * 16));
+  {
+    const int L16 = lane & 15, g16 = (lane >> 4) & 1;
+    const int r0 = 4 * hh + (L16 >> 2), r1 = r0 + 8, sub = (L16 & 1) * 8;
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db) {
+      const int chunk = 4 * db + 2 * g16 + ((L16 & 3) >> 1);
+      col_off[db][0] = (uint32_t)(r0 * ROW + ((chunk ^ swz<D>(r0)) * 16) + sub);
+      col_off[db][1] = (uint32_t)(r1 * ROW + ((chunk ^ swz<D>(r1)) * 16) + sub);
+    }
+  }
   // A operand of MFMA i of a scores phase (even i: Q rows for S, odd i: dO rows for dP) / of a gradient phase (even i:
-  // dO^T for dV, odd i: Q^T for dK)
-  auto scores_frag = [&](FO_LDS const char* qtile, FO_LDS const char* gtile, int qb, int i) -> vec8 {
-    return row_frag<T, D>((i & 1) ? gtile : qtile, qb, i >> 1, l32, hh);
+  // dO^T for dV, odd i: Q^T for dK); rq / cq = the offsets above plus the byte offset of the tile's Q buffer
+  auto scores_frag = [&](const uint32_t* rq, int qb, int i) -> vec8 {
+    return *(FO_LDS const vec8*)(smem + rq[i >> 1] + ((i & 1) ? G_OFF : 0) + qb * 32 * ROW);
   };
-  auto grads_frag = [&](FO_LDS const char* qtile, FO_LDS const char* gtile, int qb, int i) -> vec8 {
-    return col_frag<T, D>((i & 1) ? qtile : gtile, 2 * qb + i / (2 * DBLK), (i >> 1) % DBLK, lane);
+  auto grads_frag = [&](const uint32_t (*cq)[2], int qb, int i) -> vec8 {
+    const int tp = 2 * qb + i / (2 * DBLK), db = (i >> 1) % DBLK;
+    const int imm = ((i & 1) ? 0 : G_OFF) + 16 * tp * ROW;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(smem + cq[db][0] + imm));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FO_LDS s16x4*)(smem + cq[db][1] + imm));
+    return __builtin_bit_cast(vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
-  constexpr int kFragAhead = 3;
+  constexpr int kFragAhead = 4;
+  static_assert((4 * NMF) % kFragAhead == 0, "the fragment ring runs on across tiles");
   vec8 fr[kFragAhead];         // A operands, fetched kFragAhead micro-groups ahead of their MFMA
   f32x16 sacc[2], dpacc[2];
   vec8 pf[2][2], dsf[2][2];
 
   auto tile_body = [&](int j, auto masked) {
-    const int buf = (j - qt0) & 1;
+    const int buf = (j - qt0) % NBUF, nbuf = (buf + 1) % NBUF;
     const int q0t = j * kBwdTile;
-    FO_LDS const char* qtile = smem + buf * TILE_BYTES;
-    FO_LDS const char* gtile = smem + (2 + buf) * TILE_BYTES;
+    uint32_t rq[KSTEPS], cq[DBLK][2], rq_next[(kFragAhead + 1) / 2];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) { rq[ks] = row_off[ks] + (uint32_t)(buf * TILE_BYTES); asm volatile("" : "+v"(rq[ks])); }
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) { cq[db][u] = col_off[db][u] + (uint32_t)(buf * TILE_BYTES); asm volatile("" : "+v"(cq[db][u])); }
+#pragma unroll
+    for (int ks = 0; ks < (kFragAhead + 1) / 2; ++ks) { rq_next[ks] = row_off[ks] + (uint32_t)(nbuf * TILE_BYTES); asm volatile("" : "+v"(rq_next[ks])); }
     // A operand of the tile's MFMA g (phases of NMF)
     auto frag = [&](int g) -> vec8 {
       const int ph = g / NMF, i = g % NMF;
-      return ph < 2 ? scores_frag(qtile, gtile, ph, i) : grads_frag(qtile, gtile, ph - 2, i);
+      return ph < 2 ? scores_frag(rq, ph, i) : grads_frag(cq, ph - 2, i);
     };
-    auto refill = [&](int g) { if (g + kFragAhead < 4 * NMF) fr[g % kFragAhead] = frag(g + kFragAhead); };
+    // (past the end of the tile: the first fragments of the next one; read but unused after the last tile)
+    auto refill = [&](int g) {
+      fr[g % kFragAhead] = g + kFragAhead < 4 * NMF ? frag(g + kFragAhead) : scores_frag(rq_next, 0, g + kFragAhead - 4 * NMF);
+    };
     FO_LDS const float* lse_t = rowvals + buf * kBwdTile;
-    FO_LDS const float* del_t = rowvals + (2 + buf) * kBwdTile;
+    FO_LDS const float* del_t = rowvals + (NBUF + buf) * kBwdTile;
     f32x4 lv[2], dv[2];        // LSE and delta of four query rows, fetched one vector ahead
     // score element r of block qb: register r holds query q0t + 32*qb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2);
     // dead iff key > query or the query is past the end
@@ -539,15 +601,11 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       dv[0] = *(FO_LDS const f32x4*)(del_t + 32 * qb + 4 * hh);
     };
     // ---- phase 1
-#pragma unroll
-    for (int i = 0; i < kFragAhead; ++i) fr[i] = frag(i);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { sacc[0][r] = 0.0f; dpacc[0][r] = 0.0f; sacc[1][r] = 0.0f; dpacc[1][r] = 0.0f; }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = i;
-      if (i & 1) dpacc[0] = Ops<T>::mfma(fr[g % kFragAhead], vf[i >> 1], dpacc[0]); else sacc[0] = Ops<T>::mfma(fr[g % kFragAhead], kf[i >> 1], sacc[0]);
+      if (i & 1) mfma_scores_vgpr<T>(dpacc[0], fr[g % kFragAhead], vf[i >> 1], i == 1); else mfma_scores_vgpr<T>(sacc[0], fr[g % kFragAhead], kf[i >> 1], i == 0);
       refill(g);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -556,8 +614,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = NMF + i;
-      if (i & 1) dpacc[1] = Ops<T>::mfma(fr[g % kFragAhead], vf[i >> 1], dpacc[1]); else sacc[1] = Ops<T>::mfma(fr[g % kFragAhead], kf[i >> 1], sacc[1]);
+      if (i & 1) mfma_scores_vgpr<T>(dpacc[1], fr[g % kFragAhead], vf[i >> 1], i == 1); else mfma_scores_vgpr<T>(sacc[1], fr[g % kFragAhead], kf[i >> 1], i == 0);
       refill(g);
+      if (i == 0) scores_fence(sacc[0], dpacc[0]);
 #pragma unroll
       for (int e = 0; e < EPG; ++e) element(0, i * EPG + e);
       __builtin_amdgcn_sched_barrier(0);
@@ -570,10 +629,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
       if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], dsf[0][t]); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], pf[0][t]);
       refill(g);
+      if (i == 0) scores_fence(sacc[1], dpacc[1]);
 #pragma unroll
       for (int e = 0; e < EPG; ++e) element(1, i * EPG + e);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (j + 1 < n_qt) hand_over(j);
     // ---- phase 4
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
@@ -592,18 +653,17 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   // accumulator registers between homes at every tile.
   auto needs_mask = [&](int jt) { return jt * kBwdTile + kBwdTile > Sq || (CAUSAL && k0w + 31 > jt * kBwdTile); };
   j = ja;
-  for (; j < n_qt && needs_mask(j); ++j) {
-    tile_body(j, std::true_type{});
-    if (j + 1 < n_qt) hand_over(j);
+  if (j < n_qt) {
+    const int buf = (j - qt0) % NBUF;
+    uint32_t rq0[(kFragAhead + 1) / 2];
+#pragma unroll
+    for (int ks = 0; ks < (kFragAhead + 1) / 2; ++ks) rq0[ks] = row_off[ks] + (uint32_t)(buf * TILE_BYTES);
+#pragma unroll
+    for (int i = 0; i < kFragAhead; ++i) fr[i] = scores_frag(rq0, 0, i);
   }
-  for (; j < n_qt && !needs_mask(j); ++j) {
-    tile_body(j, std::false_type{});
-    if (j + 1 < n_qt) hand_over(j);
-  }
-  for (; j < n_qt; ++j) {
-    tile_body(j, std::true_type{});
-    if (j + 1 < n_qt) hand_over(j);
-  }
+  for (; j < n_qt && needs_mask(j); ++j) tile_body(j, std::true_type{});
+  for (; j < n_qt && !needs_mask(j); ++j) tile_body(j, std::false_type{});
+  for (; j < n_qt; ++j) tile_body(j, std::true_type{});
 
   acc_fence(dkacc);
   acc_fence(dvacc);
@@ -638,13 +698,14 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
   static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+  const size_t lds_pipe = 6 * (size_t)kBwdTile * D * 2 + 6 * kBwdTile * sizeof(float);   // three tile buffers
   static const hipError_t a3 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL>,
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pipe);
   if (a1 != hipSuccess || a2 != hipSuccess || a3 != hipSuccess) return FO_ERR_LAUNCH;
   attn_bwd_delta_kernel<T, D><<<(unsigned)g_delta, 256, 0, s>>>(p);
   attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(p);
   // attn_bwd.variant 0 selects the plain dK/dV kernel everywhere (tests compare the two)
-  if (!DROP && !BIAS && g_attn_bwd_variant != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
+  if (!DROP && !BIAS && g_attn_bwd_variant != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(p);
   else attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(p);
   return launch_status();
 }
