@@ -69,6 +69,43 @@ def test_attn_argument_validation_without_device():
     assert call(scale=0.0) == -4 and call(scale=-1.0) == -4
 
 
+def test_attn_backward_bias_dropout_argument_validation_without_device():
+    lib = _lib.load()
+    I3 = ctypes.c_int64 * 3
+    s = I3(128 * 64, 64 * 128 * 4, 64)
+    P = ctypes.POINTER(ctypes.c_int64)
+    strides = lambda bad=None: (P * 8)(*[ctypes.cast(bad if (bad is not None and i == 5) else s, P) for i in range(8)])
+    ok = 0x1000
+    bwd = lambda **kw: lib.fo_attn_bwd(
+        kw.get("q", ok), ok, ok, ok, ok, kw.get("lse", ok), kw.get("ws", ok), ok, ok, ok,
+        1, 1, kw.get("Sq", 128), 128, kw.get("D", 64), kw.get("strides", strides()), kw.get("scale", 0.125), 0, kw.get("dtype", 1), None)
+    assert bwd(q=None) == -1 and bwd(ws=None) == -1 and bwd(strides=None) == -1
+    assert bwd(dtype=2) == -2
+    assert bwd(D=96) == -3
+    assert bwd(Sq=0) == -4 and bwd(scale=0.0) == -4
+    assert bwd(strides=strides(I3(128 * 64, 64 * 128, 60))) == -5      # dQ rows not 16-byte aligned / shorter than D
+    assert bwd(lse=0x1002) == -6
+
+    class Extras(ctypes.Structure):
+        _fields_ = [("bias", ctypes.c_void_p), ("bias_strides", ctypes.c_int64 * 3), ("bias_dtype", ctypes.c_int),
+                    ("dropout_p", ctypes.c_float), ("dropout_seed", ctypes.c_uint32), ("dropout_offset", ctypes.c_uint64)]
+    def fwd_ex(ex):
+        return lib.fo_attn_fwd_ex(ok, ok, ok, ok, None, 1, 1, 128, 128, 64, s, s, s, s, 0.125, 0, 1, ctypes.byref(ex), None)
+    ex = Extras(); ex.bias = ok; ex.bias_strides = I3(0, 0, 128); ex.bias_dtype = 0      # fp16 bias with bf16 operands
+    assert fwd_ex(ex) == -2
+    ex.bias_dtype = 2; ex.bias_strides = I3(0, 0, -1)
+    assert fwd_ex(ex) == -5
+    ex.bias_strides = I3(0, 0, 128); ex.bias = 0x1002                                  # fp32 bias on a 2-byte boundary
+    assert fwd_ex(ex) == -6
+    ex.bias = None; ex.dropout_p = 1.0
+    assert fwd_ex(ex) == -4
+    assert lib.fo_attn_fwd_dropout(ok, ok, ok, ok, None, 1, 1, 128, 128, 64, s, s, s, s, 0.125, 0, 1, -0.1, 1, 0, None) == -4
+    assert lib.fo_dropout_mask(None, 16, 0.5, 1, 0, None) == -1
+    assert lib.fo_dropout_mask(ok, -1, 0.5, 1, 0, None) == -4
+    assert lib.fo_dropout_mask(ok, 16, 1.5, 1, 0, None) == -4
+    assert lib.fo_dropout_mask(ok, 0, 0.5, 1, 0, None) == 0                            # nothing to do, nothing launched
+
+
 def test_lion_argument_validation_without_device():
     lib = _lib.load()
     c = _lib.FoLionConsts()
