@@ -18,9 +18,13 @@
 //      computed untransposed, S = Q K^T and dP = dO V^T (A operands = Q / dO rows from LDS, B operands = K^T / V^T
 //      held in registers), so a lane owns one key and P, dS are the B operands of dV^T = dO^T P and dK^T = Q^T dS
 //      (A operands via the transposing LDS read of the dO and Q tiles); per-row LSE and delta come from LDS.
-// Both recompute the scores (seven GEMMs in total instead of the five of an atomics-based single pass).
-// Tiles of 64 rows go global -> LDS with the direct-to-LDS loads, double buffered, one barrier per tile, 16-byte
-// chunks XOR-swizzled inside a row (no bank conflicts), exactly as in the 128-row forward kernel.
+//      Without dropout and bias this runs as attn_bwd_dkdv_pipe_kernel, the same computation laid out by hand as a
+//      software pipeline (described there); attn_bwd_dkdv_kernel is the plain, compiler-scheduled form.
+// Both recompute the scores (seven GEMMs in total instead of the five of an atomics-based single pass). softmax_scale
+// is applied once to the finished dQ and dK accumulators rather than to every dS.
+// Tiles of 64 rows go global -> LDS with the direct-to-LDS loads, double buffered (three buffers in the pipelined
+// kernel), one barrier per tile, 16-byte chunks XOR-swizzled inside a row (no bank conflicts), exactly as in the
+// 128-row forward kernel.
 #include <type_traits>
 
 #include "attn_common.hpp"
