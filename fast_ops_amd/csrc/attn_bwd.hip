@@ -151,6 +151,33 @@ __device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int r
   }
 }
 
+// The same copy for a tile that lies wholly inside the matrix, with the address split into a wave-uniform base (the
+// tile's first row: scalar arithmetic, once per tile) and per-lane byte offsets that never change (TileLaneOffsets,
+// computed once per kernel): two instructions per 1 KiB piece instead of a 64-bit multiply-add per lane and piece.
+template <typename T, int D>
+struct TileLaneOffsets {
+  static constexpr int N = kBwdTile * D * 2 / 1024 / kBwdWaves;   // pieces per wave and tile
+  uint32_t off[N];
+  bool ok;                                                        // 32-bit offsets suffice for this row stride
+  __device__ __forceinline__ void init(int64_t stride, int wave_s, int lane) {
+    constexpr int ROW_BYTES = D * 2, CHUNKS = ROW_BYTES / 16, ROWS_PER_DMA = 1024 / ROW_BYTES;
+    ok = stride < (1 << 23);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int row = (wave_s * N + i) * ROWS_PER_DMA + lane / CHUNKS;
+      const int col = ((lane % CHUNKS) ^ swz<D>(row)) * 8;
+      off[i] = (uint32_t)(row * (int)stride + col) * 2u;
+    }
+  }
+};
+template <typename T, int D>
+__device__ __forceinline__ void copy_tile64_inside(const T* base, int64_t stride, int row0, const TileLaneOffsets<T, D>& lo,
+                                                   FO_LDS char* dst, int wave_s) {
+  const char* tile = (const char*)(base + (int64_t)row0 * stride);
+#pragma unroll
+  for (int i = 0; i < TileLaneOffsets<T, D>::N; ++i) dma16_uniform_base(tile, lo.off[i], dst + (wave_s * TileLaneOffsets<T, D>::N + i) * 1024);
+}
+
 // A operand of a 32x32x16 MFMA from a row-major tile in LDS: lane = row l32 of block `blk`, 8 elements at
 // column 16*ks + 8*hh
 template <typename T, int D>
@@ -327,9 +354,17 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   const int n_qt = (Sq + kBwdTile - 1) / kBwdTile;
   const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;   // queries before the block's first key never attend it
 
+  TileLaneOffsets<T, D> qlo, glo;
+  qlo.init(prm.qs[2], wave_s, lane);
+  glo.init(prm.dos[2], wave_s, lane);
   auto issue = [&](int qt, int buf) {
-    copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
-    copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    if (qt * kBwdTile + kBwdTile <= Sq && qlo.ok && glo.ok) {
+      copy_tile64_inside<T, D>(qbase, prm.qs[2], qt * kBwdTile, qlo, smem + buf * TILE_BYTES, wave_s);
+      copy_tile64_inside<T, D>(gbase, prm.dos[2], qt * kBwdTile, glo, smem + (2 + buf) * TILE_BYTES, wave_s);
+    } else {
+      copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    }
     // per-row LSE and delta of the tile, 4 bytes per lane, also straight into LDS (a load the compiler can see would
     // make it wait for the tile copies as well); rows past the end re-read the last row and are masked below
     if (wave_s < 2) {
@@ -483,9 +518,17 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;     // queries before the block's first key never attend it
   const int ja = CAUSAL ? min(k0w / kBwdTile, n_qt) : 0;     // ... and this wave's keys start later still
 
+  TileLaneOffsets<T, D> qlo, glo;
+  qlo.init(prm.qs[2], wave_s, lane);
+  glo.init(prm.dos[2], wave_s, lane);
   auto issue = [&](int qt, int buf) {
-    copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
-    copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (NBUF + buf) * TILE_BYTES, wave_s, lane);
+    if (qt * kBwdTile + kBwdTile <= Sq && qlo.ok && glo.ok) {
+      copy_tile64_inside<T, D>(qbase, prm.qs[2], qt * kBwdTile, qlo, smem + buf * TILE_BYTES, wave_s);
+      copy_tile64_inside<T, D>(gbase, prm.dos[2], qt * kBwdTile, glo, smem + (NBUF + buf) * TILE_BYTES, wave_s);
+    } else {
+      copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (NBUF + buf) * TILE_BYTES, wave_s, lane);
+    }
     if (wave_s < 2) {
       const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
       dma4_lane_ptr((wave_s == 0 ? prm.lse : (const float*)prm.delta) + at, rowvals + (NBUF * wave_s + buf) * kBwdTile);
