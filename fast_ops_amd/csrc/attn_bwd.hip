@@ -137,7 +137,11 @@ __global__ void __launch_bounds__(256) attn_bwd_delta_kernel(const AttnBwdParams
 // back to back, so the swizzle is applied by choosing which global chunk a lane fetches. Rows past the end re-read
 // the last row (callers mask them).
 template <typename T, int D>
-__device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int row0, int S, FO_LDS char* dst, int wave_s, int lane) {
+__device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int row0, int S, FO_LDS char* dst, int wave_s, int lane_in) {
+  // (an opaque copy of the lane index: this is the path of tiles that cross the end of the matrix, taken once per
+  // workgroup at most; its address arithmetic must not be hoisted out of it into registers that live across the loop)
+  int lane = lane_in;
+  asm volatile("" : "+v"(lane));
   constexpr int ROW_BYTES = D * 2;
   constexpr int CHUNKS = ROW_BYTES / 16;
   constexpr int ROWS_PER_DMA = 1024 / ROW_BYTES;
@@ -222,9 +226,17 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   const T* vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
   const int n_tiles = CAUSAL ? (min(Sk, q0 + kBwdRows) + kBwdTile - 1) / kBwdTile : (Sk + kBwdTile - 1) / kBwdTile;
 
+  TileLaneOffsets<T, D> klo, vlo;
+  klo.init(prm.ks[2], wave_s, lane);
+  vlo.init(prm.vs[2], wave_s, lane);
   auto issue = [&](int tile, int buf) {
-    copy_tile64<T, D>(kbase, prm.ks[2], tile * kBwdTile, Sk, smem + buf * TILE_BYTES, wave_s, lane);
-    copy_tile64<T, D>(vbase, prm.vs[2], tile * kBwdTile, Sk, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    if (tile * kBwdTile + kBwdTile <= Sk && klo.ok && vlo.ok) {
+      copy_tile64_inside<T, D>(kbase, prm.ks[2], tile * kBwdTile, klo, smem + buf * TILE_BYTES, wave_s);
+      copy_tile64_inside<T, D>(vbase, prm.vs[2], tile * kBwdTile, vlo, smem + (2 + buf) * TILE_BYTES, wave_s);
+    } else {
+      copy_tile64<T, D>(kbase, prm.ks[2], tile * kBwdTile, Sk, smem + buf * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(vbase, prm.vs[2], tile * kBwdTile, Sk, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+    }
   };
   issue(0, 0);
 
