@@ -18,11 +18,12 @@
 //   * K/V tiles (64 keys) go global -> LDS with the direct-to-LDS loads (16 B per lane, no VGPR staging).
 //   * Workgroup order: heads are dealt to the 8 XCDs (workgroup ids round-robin over XCDs), each XCD walks one head
 //     at a time, so an XCD's L2 holds the K/V it is streaming.
-// attn_fwd_kernel (head_dim 64, and head_dim 128 for small or very long inputs): one workgroup = 4 waves = 128 query
+// attn_fwd_kernel (small or very long inputs; bias and dropout): one workgroup = 4 waves = 128 query
 //   rows, two workgroups per CU, compiler-scheduled MFMA builtins, tiles double buffered with one barrier per tile,
 //   16-byte chunks XOR-swizzled inside a row so that both the K reads (32 rows x one chunk) and the V reads (4 rows x
 //   4 chunks) are free of bank conflicts; heaviest (last) causal query blocks first.
-// attn_fwd_wide_kernel (head_dim 128): 256 query rows per workgroup, one workgroup per CU, MFMAs as inline assembly
+// attn_fwd_wide_kernel (the default once a shape gives every CU a workgroup): 256 query rows per workgroup, one
+//   workgroup per CU (two fit for head_dim 64), MFMAs as inline assembly
 //   with the accumulators of O and the fragments of Q in AGPRs, a three-deep software pipeline over 32-key sub-tiles
 //   laid out as micro-groups of one MFMA plus its share of everything else; described where it is defined.
 #include <type_traits>
@@ -654,13 +655,16 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     constexpr int P = decltype(parity)::value;
     constexpr bool HAS_QK = decltype(has_qk)::value, HAS_PV = decltype(has_pv)::value, MASK = decltype(masked)::value;
     constexpr int NM = QB * KSTEPS;                                     // MFMAs of one kind
-    constexpr int G = (HAS_QK ? NM : 0) + (HAS_PV ? NM : 0);            // micro-groups
+    constexpr int NMF = (HAS_QK ? NM : 0) + (HAS_PV ? NM : 0);          // micro-groups with an MFMA
     constexpr int NEL = 16 * QB;                                        // scores per lane
     // Group 0 only issues its MFMA: the scores of this sub-tile were written by MFMAs up to the last-but-one group of
     // the previous step. Then the mask (if any), then the exponentials.
     constexpr int GMASK = 1;
     constexpr int GE0 = MASK ? 2 : 1;                                   // first group that may read the scores
     constexpr int DA = 1;                                               // groups between an exponential and its use
+    // (a step with few MFMAs - head_dim 64, first or last step - gets groups without one, so that the three stages of
+    // the softmax arithmetic still have their places)
+    constexpr int G = NMF > GE0 + 3 + DA ? NMF : GE0 + 3 + DA;          // micro-groups
     constexpr int NE = G - 1 - DA - GE0;                                // groups GE0+1 .. G-1-DA carry the exponentials
     static_assert(NE >= 2, "too few micro-groups");
     // (an opaque copy of the sub-tile index: the variants of this step are selected by branches, and identical address
@@ -683,7 +687,8 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       const bool is_qk = HAS_QK && (!HAS_PV || (g & 1) == 0);
       const int i = (HAS_QK && HAS_PV) ? (g >> 1) : g;                 // index among the MFMAs of its kind
       const int f = i / QB, qb = i % QB;                               // fragment, query block
-      if (is_qk) {
+      if (g >= NMF) {
+      } else if (is_qk) {
         if (f == 0) Mfma::v_init_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
         else Mfma::v_acc_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
         if (qb == QB - 1 && !(DBG & 4)) KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb1, f + RD) : k_frag(kb2, f + RD - KSTEPS);
@@ -953,15 +958,19 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
     return causal ? launch_one<T, D, true, true, 0, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, true>(p, stream);
   }
   if (dropout) return causal ? launch_one<T, D, true, true, 0, true>(p, stream) : launch_one<T, D, false, true, 0, true>(p, stream);
-  // default: the wide kernel (eight waves x 32 rows) for head_dim 128, the 128-row kernel for head_dim 64
-  // (the wide kernel addresses a head's keys with 32-bit byte offsets)
+  // default: the wide kernel (eight waves x 32 rows)
+  // (it addresses a head's keys with 32-bit byte offsets)
   // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
   // 128-row kernel, with four times as many workgroups, fills the chip better
   static const int n_cu = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256; return n; }();
   const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
-  const bool wide_ok = D == 128 && (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
+  const bool wide_ok = (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
   int v = g_attn_variant < 0 ? (wide_ok && wide_wgs >= n_cu ? 16 : 0) : g_attn_variant;
   if (!wide_ok && v >= 16) v = 0;
+  if constexpr (D == 64) {
+    if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
+    if (v >= 16) v = 0;
+  }
   if constexpr (D == 128) {
     // 16: wide kernel, eight waves x 32 rows; 32: wide kernel, four waves x 64 rows
     if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);

@@ -41,7 +41,7 @@ def _check(o, lse, o_ref, lse_ref, what=""):
 
 
 # attn.variant values: -1 = the library's choice (which depends on head_dim and on how many workgroups the shape gives),
-# 0 = the 128-row kernel, 16 / 32 = the 256-row kernel with eight / four waves (head_dim 128 only)
+# 0 = the 128-row kernel, 16 / 32 = the 256-row kernel with eight / four waves (four: head_dim 128 only)
 KERNELS_D128 = [-1, 0, 16, 32]
 
 
@@ -94,8 +94,8 @@ def test_throughput_shape_slice_fp16_noncausal():
 @pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
 def test_ragged_and_unequal_lengths(shape, causal, D, kernel_variant):
     # sequence lengths that are not multiples of the 128-row / 64-key tiles, Sq != Sk (causal mask is top-left aligned)
-    if D == 64 and kernel_variant > 0:
-        pytest.skip("head_dim 64 has one kernel")
+    if D == 64 and kernel_variant == 32:
+        pytest.skip("head_dim 64 has no four-wave form of the 256-row kernel")
     B, H, Sq, Sk = shape
     _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
 
@@ -110,14 +110,28 @@ def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype, kerne
     _run_and_check(B, H, Sq, Sk, 128, dtype, causal, seed=Sq + Sk)
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("kernel_variant", [-1, 0, 16], indirect=True)
+def test_ragged_across_256_row_blocks_head_dim_64(shape, causal, dtype, kernel_variant):
+    B, H, Sq, Sk = shape
+    _run_and_check(B, H, Sq, Sk, 64, dtype, causal, seed=Sq + Sk + 64)
+
+
+def test_head_dim_64_large_shape_takes_the_256_row_kernel_by_default():
+    # enough 256-row workgroups for every CU: the library's own choice must agree with the oracle too
+    _run_and_check(2, 40, 2048, 2048, 64, torch.bfloat16, True, seed=5)
+
+
 @pytest.mark.parametrize("pattern", ["growing", "shrinking", "spikes"])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
 @pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
 def test_moving_row_maximum(pattern, causal, D, dtype, kernel_variant):
-    if D == 64 and kernel_variant > 0:
-        pytest.skip("head_dim 64 has one kernel")
+    if D == 64 and kernel_variant == 32:
+        pytest.skip("head_dim 64 has no four-wave form of the 256-row kernel")
     # scores whose row maximum keeps moving (or sits far above the rest) exercise the rescaling of the running
     # softmax state: keys scaled so that scaled scores span tens of units
     B, H, Sq, Sk = 1, 2, 384, 640
