@@ -818,6 +818,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   p.bias.ptr = bias;
   for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
   p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
+  p.bias.dma_ok = 0;   // (the backward kernels read the bias element by element)
 #define FO_BWD2(T, DD, BI) (drop ? (c ? launch_bwd<T, DD, true, true, BI>(p, s) : launch_bwd<T, DD, false, true, BI>(p, s)) \
                                  : (c ? launch_bwd<T, DD, true, false, BI>(p, s) : launch_bwd<T, DD, false, false, BI>(p, s)))
 #define FO_BWD(T, DD) (bias ? FO_BWD2(T, DD, true) : FO_BWD2(T, DD, false))

@@ -79,6 +79,7 @@ struct BiasParams {
   const void* ptr;
   int64_t strides[3];
   int is_f32;
+  int dma_ok;   // base and the three strides are multiples of 16 bytes: tiles may be copied with 16-byte pieces
 };
 template <typename T>
 __device__ __forceinline__ float load_bias(const BiasParams& bp, int64_t at) {

@@ -148,7 +148,35 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     }
   };
 
+  // ---- bias: the wave's 32 query rows x 64 keys of a tile, copied like K and V straight into LDS (a per-lane global
+  // read of "my row" touches 64 cache lines per instruction). Two buffers of 8 KiB per wave behind the K/V tiles. A row
+  // of the tile is 256 bytes (fp32) or 128 bytes (operand type) = 16 or 8 pieces of 16 bytes; piece s of LDS row r
+  // holds the row's piece s ^ (r mod 16 or 8), so the reads below (32 rows x the same piece) are spread over the banks.
+  // Only for complete tiles of suitably aligned tensors; everything else takes the per-element loads further down.
+  constexpr int kBiasWaveBytes = 32 * kBN * 4;
+  FO_LDS char* bias_lds = smem + 4 * TILE_BYTES + wave_s * kBiasWaveBytes;
+  auto issue_bias = [&](int tile, int buf) {
+    if (!prm.bias.dma_ok || tile * kBN + kBN > Sk) return;
+    int lane_here = lane;                      // (opaque: this arithmetic is redone per tile rather than kept in registers)
+    asm volatile("" : "+v"(lane_here));
+    const int elt = prm.bias.is_f32 ? 4 : 2;
+    const int pieces = prm.bias.is_f32 ? 16 : 8, rows_per_dma = 64 / pieces;
+    const char* base = (const char*)prm.bias.ptr + (b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)tile * kBN) * elt;
+    FO_LDS char* dst = bias_lds + buf * kWaves * kBiasWaveBytes;
+    const int n_dma = prm.bias.is_f32 ? 8 : 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i < n_dma) {
+        const int row = i * rows_per_dma + lane_here / pieces;
+        const int piece = (lane_here % pieces) ^ (row & (pieces - 1));
+        const int64_t q = min(q0w + row, Sq - 1);
+        dma16_lane_ptr(base + q * prm.bias.strides[2] * elt + piece * 16, dst + i * 1024);
+      }
+    }
+  };
+
   issue_tile(0, 0);
+  if constexpr (BIAS) issue_bias(0, 0);
 
   // ---- Q^T fragments (B operand): lane holds query row q0w + l32, d = 16*ks + 8*hh .. +7
   vec8 qf[KSTEPS];
@@ -186,6 +214,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's pieces of tile `tile` have landed in LDS
     if (!(DBG & 4)) __syncthreads();        // everyone's pieces have landed; everyone is done reading the other buffer
     if (tile + 1 < n_tiles && (!(DBG & 1) || tile < 1)) issue_tile(tile + 1, buf ^ 1);
+    if constexpr (BIAS) { if (tile + 1 < n_tiles) issue_bias(tile + 1, buf ^ 1); }
 
     // waves whose rows are all above this tile's keys have nothing to do (causal)
     if (CAUSAL && key0 > q0w + 31) continue;
@@ -242,15 +271,38 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     }
 
     if constexpr (BIAS) {
-      // qk * softmax_scale + bias (flash_attention_triton.py:198); rows and keys past the end re-read the last ones
-      const int64_t brow = b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)min(q0w + l32, Sq - 1) * prm.bias.strides[2];
+      // qk * softmax_scale + bias (flash_attention_triton.py:198)
+      if (prm.bias.dma_ok && key0 + kBN <= Sk) {
+        // from the tile copied into LDS: register r = 4 j + u of block kb is key 32 kb + 8 j + 4 hh + u of row l32
+        FO_LDS const char* bt = bias_lds + buf * kWaves * kBiasWaveBytes;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = min(key0 + 32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2), Sk - 1);
-          sacc[kb][r] = __builtin_fmaf(sacc[kb][r], prm.scale_log2e, load_bias<T>(prm.bias, brow + key) * 1.4426950408889634f);
-        }
+          for (int j = 0; j < 4; ++j) {
+            f32x4 bv;
+            if (prm.bias.is_f32) {
+              bv = *(FO_LDS const f32x4*)(bt + l32 * 256 + (((8 * kb + 2 * j + hh) ^ (l32 & 15)) * 16));
+            } else {
+              typedef __attribute__((ext_vector_type(4))) T vec4;
+              const vec4 h4 = *(FO_LDS const vec4*)(bt + l32 * 128 + (((4 * kb + j) ^ (l32 & 7)) * 16) + hh * 8);
+#pragma unroll
+              for (int u = 0; u < 4; ++u) bv[u] = (float)h4[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              sacc[kb][4 * j + u] = __builtin_fmaf(sacc[kb][4 * j + u], prm.scale_log2e, bv[u] * 1.4426950408889634f);
+          }
+      } else {
+        // per-element loads; rows and keys past the end re-read the last ones
+        const int64_t brow = b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)min(q0w + l32, Sq - 1) * prm.bias.strides[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = min(key0 + 32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2), Sk - 1);
+            sacc[kb][r] = __builtin_fmaf(sacc[kb][r], prm.scale_log2e, load_bias<T>(prm.bias, brow + key) * 1.4426950408889634f);
+          }
+      }
     }
 
     // ---- online softmax (base-2 domain) with a lazily updated reference maximum.
@@ -939,10 +991,11 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
 
 template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false>
 static int launch_one(const AttnParams& p, hipStream_t stream) {
-  const size_t lds = 4 * (size_t)kBN * D * 2;
+  const size_t lds_max = 4 * (size_t)kBN * D * 2 + (BIAS ? 2 * kWaves * 32 * kBN * 4 : 0);   // K, V tiles; bias tiles
+  const size_t lds = 4 * (size_t)kBN * D * 2 + (BIAS && p.bias.dma_ok ? 2 * kWaves * 32 * kBN * 4 : 0);
   const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
   static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
   attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS><<<grid, kWaves * 64, lds, stream>>>(p);
   return launch_status();
@@ -1055,6 +1108,13 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   p.bias.ptr = bias;
   for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
   p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
+  {
+    const int64_t elt = p.bias.is_f32 ? 4 : 2;
+    // (a bias that is the same for every query - query stride 0 - is one row per tile: per-element loads of it are
+    // broadcasts, and the kernel keeps its two workgroups per CU without the LDS for bias tiles)
+    p.bias.dma_ok = bias && p.bias.strides[2] != 0 && ((uintptr_t)bias % 16) == 0 && (p.bias.strides[0] * elt) % 16 == 0 &&
+                    (p.bias.strides[1] * elt) % 16 == 0 && (p.bias.strides[2] * elt) % 16 == 0;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == FO_DTYPE_BF16) return D == 128 ? launch<__bf16, 128>(p, causal != 0, drop, s) : launch<__bf16, 64>(p, causal != 0, drop, s);
   return D == 128 ? launch<_Float16, 128>(p, causal != 0, drop, s) : launch<_Float16, 64>(p, causal != 0, drop, s);

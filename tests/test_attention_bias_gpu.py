@@ -51,6 +51,31 @@ def test_bias_shapes_of_the_reference(D, kind, causal, dtype):
     _check(_bshd(o), lse, [_bshd(t) for t in got], o_ref, lse_ref, ref)
 
 
+@pytest.mark.parametrize("bias_dtype", ["f32", "operand"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["1h1k", "1hqk", "b11k", "bhqk"])
+@pytest.mark.parametrize("shape", [(200, 320, 128), (130, 200, 64), (64, 64, 128), (300, 1032, 64)])
+def test_bias_rows_on_16_byte_boundaries(shape, kind, causal, bias_dtype):
+    # key counts that put every bias row on a 16-byte boundary: complete 64-key tiles of the bias then reach the forward
+    # kernel through its tile copies (the last, partial tile and every other alignment through per-element loads)
+    Sq, Sk, D = shape
+    B, H, dtype = 2, 2, torch.bfloat16
+    g = torch.Generator().manual_seed(Sq + Sk)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk, Sq))
+    bias = _bias(kind, B, H, Sq, Sk, torch.float32 if bias_dtype == "f32" else dtype, g) * 2.0
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, bias=bias)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal, bias=bias)
+    qd, kd, vd = (_bshd(t.to(DEV)).requires_grad_(True) for t in (q, k, v))
+    o, lse = flash_attn(qd, kd, vd, bias=bias.to(DEV), causal=causal, return_lse=True)
+    got = torch.autograd.grad(o, (qd, kd, vd), _bshd(go.to(DEV)))
+    _check(_bshd(o), lse, [_bshd(t) for t in got], o_ref, lse_ref, ref)
+    # a view whose rows do not start on 16-byte boundaries gives the same result through the other path
+    shifted = torch.empty(bias.shape[:-1] + (Sk + 1,), dtype=bias.dtype, device=DEV)[..., 1:]
+    shifted.copy_(bias)
+    o2 = flash_attn(qd, kd, vd, bias=shifted, causal=causal)
+    assert torch.equal(o2, o)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
 @pytest.mark.parametrize("kind", ["1h1k", "b1qk"])
 def test_bias_in_the_operand_dtype(kind, dtype):
