@@ -81,6 +81,21 @@ def test_long_sequence_many_tiles_per_key_block(causal, dkdv_variant):
     _run(1, 2, 1024, 1024, 128, torch.bfloat16, causal, seed=11)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_long_context_slice_of_headline_shape(causal, dkdv_variant):
+    # one (batch, head) slice of the benchmark shape S=8192 D=128 bf16 against the fp32 closed form: 128 query tiles per
+    # key block, the last ones far behind the first. Absolute criterion (the half-precision PyTorch yardstick of the
+    # other tests takes minutes on a CPU at this size): error within 2 % of the gradient's largest magnitude.
+    q, k, v, go = _inputs(1, 1, 8192, 8192, 128, torch.bfloat16, seed=8192)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o = multi_head_attention(qd, kd, vd, causal=causal)
+    got = torch.autograd.grad(o, (qd, kd, vd), go.to(DEV))
+    for name, a, r in zip(("dQ", "dK", "dV"), got, ref):
+        e = (a.float().cpu() - r).abs().max().item()
+        assert math.isfinite(e) and e <= 2e-2 * max(1.0, r.abs().max().item()), f"{name}: error {e:.3e} vs magnitude {r.abs().max().item():.3e}"
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 300),
                                    (1, 1, 300, 64), (2, 2, 191, 191), (1, 1, 385, 513)])
 @pytest.mark.parametrize("causal", [False, True])
