@@ -5,7 +5,8 @@
 Prints ONE JSON line. The headline value is the attention forward throughput at B=2 H=16 S=8192 D=128 bf16 causal
 (FLOPs counted as 2*B*H*S^2*D); the fused Lion step over 1,308,622,848 fp32 parameters with bf16 momentum (16 bytes
 per parameter) is reported in the "lion" object of the same line, each with its roofline and a CPU baseline timed on
-this host's cores. The attention backward of the same shape is reported in "attn_bwd".
+this host's cores. The attention backward of the same shape is reported in "attn_bwd", and the rate of the vendor
+library's plain bf16 GEMM on random operands on the same box in "library_gemm" (what MFMA code reaches here at all).
 """
 import argparse
 import json
@@ -98,6 +99,17 @@ def bench_attention(steps, warmup, cpu_baseline):
                      "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "flops_per_launch": bwd_flops},
         "workload": "attention bwd (delta + dQ + dK/dV kernels) of the same shape, FLOPs by the five-GEMM count",
     }
+    # yardstick, not part of the headline: the vendor library's plain bf16 GEMM on the same box with the same kind of
+    # data. Under a full-chip MFMA load the clock follows the power drawn, which depends on the operand bits (all-zero
+    # operands run a third faster than random ones), so the published peak is not what random data can reach.
+    n = 8192
+    ga, gb = (torch.randn(n, n, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
+    _, g_kernel, _ = _time_steps(lambda: torch.matmul(ga, gb), 20, 20)
+    res["library_gemm"] = {
+        "value": 2.0 * n ** 3 / (g_kernel * 1e-3) / 1e12, "unit": "TFLOP/s", "frac_of_peak": 2.0 * n ** 3 / (g_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
+        "what": f"torch.matmul (hipBLASLt) bf16 {n}x{n}x{n}, standard normal operands, same box, timed after the attention runs",
+    }
+    del ga, gb
     if cpu_baseline:
         # bounded sample: all (batch, head) slices of the same workload through the oracle's fp32 vanilla path on all host
         # cores, stopped after about 15 s; the rate is that of the slices that were finished
@@ -225,6 +237,8 @@ def main():
         line["lion"] = {k: v for k, v in lion.items() if k != "workload"}
     if attn is not None and "bwd" in attn:
         line["attn_bwd"] = attn["bwd"]
+    if attn is not None and "library_gemm" in attn:
+        line["library_gemm"] = attn["library_gemm"]
     print(json.dumps(line))
 
 
