@@ -7,6 +7,8 @@ namespace fo {
 int g_lion_variant = -1;
 int g_attn_variant = -1;
 int g_attn_bwd_variant = -1;
+int g_attn_order = -1;
+int g_attn_bwd_order = -1;
 }  // namespace fo
 
 extern "C" const char* fo_strerror(int status) {
@@ -32,6 +34,8 @@ extern "C" int fo_tune_set(const char* key, int value) {
   if (strcmp(key, "lion.variant") == 0) { fo::g_lion_variant = value; return FO_OK; }
   if (strcmp(key, "attn.variant") == 0) { fo::g_attn_variant = value; return FO_OK; }
   if (strcmp(key, "attn_bwd.variant") == 0) { fo::g_attn_bwd_variant = value; return FO_OK; }
+  if (strcmp(key, "attn.order") == 0) { fo::g_attn_order = value; return FO_OK; }
+  if (strcmp(key, "attn_bwd.order") == 0) { fo::g_attn_bwd_order = value; return FO_OK; }
   return FO_ERR_UNSUPPORTED;
 }
 
@@ -40,5 +44,7 @@ extern "C" int fo_tune_get(const char* key) {
   if (strcmp(key, "lion.variant") == 0) return fo::g_lion_variant;
   if (strcmp(key, "attn.variant") == 0) return fo::g_attn_variant;
   if (strcmp(key, "attn_bwd.variant") == 0) return fo::g_attn_bwd_variant;
+  if (strcmp(key, "attn.order") == 0) return fo::g_attn_order;
+  if (strcmp(key, "attn_bwd.order") == 0) return fo::g_attn_bwd_order;
   return FO_ERR_UNSUPPORTED;
 }

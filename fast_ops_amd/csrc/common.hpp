@@ -22,6 +22,8 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 extern int g_lion_variant;
 extern int g_attn_variant;
 extern int g_attn_bwd_variant;
+extern int g_attn_bwd_order;   // attention backward: -1 automatic, 0 all heads in one group, n > 0 groups of n heads
+extern int g_attn_order;   // 128-row attention kernel, causal: -1 automatic, 0 head by head, n > 0 heaviest query blocks first within groups of n heads per XCD
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? FO_OK : FO_ERR_LAUNCH; }
 

@@ -81,6 +81,21 @@ def test_long_sequence_many_tiles_per_key_block(causal, dkdv_variant):
     _run(1, 2, 1024, 1024, 128, torch.bfloat16, causal, seed=11)
 
 
+@pytest.mark.parametrize("group", [-1, 0, 3, 8, 16, 1000])
+@pytest.mark.parametrize("heads", [(4, 5), (3, 8)])
+def test_workgroup_order_head_groups(group, heads):
+    # attn_bwd.order: how many heads form a group in the order of the workgroups of the dQ and dK/dV kernels (0: all,
+    # -1: the library's choice). Every (head, block) must be computed exactly once whatever the grouping, also when the
+    # last group is smaller than the others (20 heads in groups of 3, 8 or 16).
+    from fast_ops_amd import _lib
+    B, H = heads
+    _lib.tune_set("attn_bwd.order", group)
+    try:
+        _run(B, H, 300, 300, 64, torch.bfloat16, True, seed=21)
+    finally:
+        _lib.tune_set("attn_bwd.order", -1)
+
+
 @pytest.mark.parametrize("causal", [True, False])
 def test_long_context_slice_of_headline_shape(causal, dkdv_variant):
     # one (batch, head) slice of the benchmark shape S=8192 D=128 bf16 against the fp32 closed form: 128 query tiles per

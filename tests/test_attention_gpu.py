@@ -71,6 +71,23 @@ def test_config2_gpt2_small_bf16_causal():
     _run_and_check(8, 12, 1024, 1024, 64, torch.bfloat16, True, seed=0, scale=0.125)
 
 
+@pytest.mark.parametrize("group", [-1, 0, 1, 2, 3, 5, 1000])
+@pytest.mark.parametrize("heads", [(2, 4), (5, 8), (3, 5)])
+def test_causal_workgroup_order_of_128_row_kernel(group, heads):
+    # attn.order: how many of an XCD's heads form a group whose heaviest query blocks run first (0: head by head, -1:
+    # the library's choice). Every (head, query block) must be computed exactly once whatever the grouping, also when
+    # the last group is smaller than the others (40 heads = 5 per XCD in groups of 2 or 3) and when the number of heads
+    # is no multiple of the 8 XCDs (15 heads: the grouping does not apply).
+    B, H = heads
+    _lib.tune_set("attn.variant", 0)
+    _lib.tune_set("attn.order", group)
+    try:
+        _run_and_check(B, H, 700, 700, 64, torch.bfloat16, True, seed=11)
+    finally:
+        _lib.tune_set("attn.variant", -1)
+        _lib.tune_set("attn.order", -1)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
