@@ -315,11 +315,29 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
         const int key_base = key0 + 32 * kb + 4 * hh;
         int lim = key_base - Sk + 1;
         if (CAUSAL) lim = max(lim, key_base - (q0w + l32));
+        // the bias of this lane's 16 keys: four loads of four consecutive keys when the tile is complete and the
+        // bias is laid out for it, else key by key (every lane reads its own row: an instruction touches 32 cache
+        // lines either way, so fewer instructions is what counts)
+        float bv[BIAS ? 16 : 1];
+        if constexpr (BIAS) {
+          if (prm.bias.vec_ok && key0 + kBwdTile <= Sk) {
+            if (prm.bias.is_f32) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) load_bias4<float>((const float*)prm.bias.ptr + bias_row + key_base + 8 * j, bv + 4 * j);
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) load_bias4<T>((const T*)prm.bias.ptr + bias_row + key_base + 8 * j, bv + 4 * j);
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bv[r] = load_bias<T>(prm.bias, bias_row + min(key_base + (r & 3) + 8 * (r >> 2), Sk - 1));
+          }
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const bool dead = decltype(masked)::value && lim > -((r & 3) + 8 * (r >> 2));
           float shift = -lse2;
-          if constexpr (BIAS) shift = __builtin_fmaf(load_bias<T>(prm.bias, bias_row + min(key_base + (r & 3) + 8 * (r >> 2), Sk - 1)), kLog2e, -lse2);
+          if constexpr (BIAS) shift = __builtin_fmaf(bv[r], kLog2e, -lse2);
           const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, shift));
           float dp = dpacc[kb][r];
           if constexpr (DROP) {
@@ -363,7 +381,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   constexpr int KSTEPS = D / 16;
   constexpr int DBLK = D / 32;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q0 | Q1 | dO0 | dO1 | lse[2][64] | delta[2][64]
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q0 | Q1 | dO0 | dO1 | lse[2][64] | delta[2][64] | bias tiles (BIAS)
   FO_LDS float* rowvals = (FO_LDS float*)(smem + 4 * TILE_BYTES);
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -382,7 +400,46 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   TileLaneOffsets<T, D> qlo, glo;
   qlo.init(prm.qs[2], wave_s, lane);
   glo.init(prm.dos[2], wave_s, lane);
+  // ---- bias. A lane owns a key and its registers run over queries, so a bias that is the same for every query (query
+  // stride 0) is one value per lane for the whole kernel. Otherwise the wave's 64 queries x 32 keys of a tile are
+  // copied straight into LDS together with the tile (a load the compiler can see is waited for right where it is
+  // issued, together with the tile copies in flight, which then no longer overlap the arithmetic): two buffers of
+  // kBiasWaveBytes per wave. A row of the wave's part is 128 bytes (fp32) or 64 bytes (operand type), so one copy
+  // instruction of 64 x 16 bytes holds 8 or 16 rows; inside it, row 4*hh + u (+ 8 for the second eight) sits in
+  // slot 2*u + hh (+ 8), so that a lane reads register u at a fixed distance from its base and the two halves of
+  // a wave, four rows apart, read different banks. Only complete tiles of suitably aligned tensors; the rest reads
+  // the bias element by element.
+  constexpr int kBiasWaveBytes = kBwdTile * 32 * 4;
+  FO_LDS char* bias_lds = (FO_LDS char*)(rowvals + 4 * kBwdTile) + wave_s * 2 * kBiasWaveBytes;
+  const bool bias_per_key = BIAS && prm.bias.strides[2] == 0;
+  const bool bias_staged = BIAS && !bias_per_key && prm.bias.dma_ok && k0 + wave_s * 32 + 32 <= Sk &&
+                           prm.bias.strides[2] > 0 && prm.bias.strides[2] < (1 << 24);   // (32-bit offsets inside a copy instruction)
+  float bias_lane = 0.0f;
+  if (bias_per_key) bias_lane = load_bias<T>(prm.bias, b * prm.bias.strides[0] + h * prm.bias.strides[1] + min(k0w + l32, Sk - 1)) * kLog2e;
+  // (per lane: the byte offset of its piece inside the rows of one copy instruction, added to a uniform base per
+  // instruction. Handing base and offset to the copy separately, as a scalar base plus a 32-bit lane offset, left the
+  // GPU faulted in this kernel for a reason not found; the per-lane 64-bit pointer is the form that is tested.)
+  uint32_t bias_lane_off = 0;
+  const char* bias_src = nullptr;
+  int64_t bias_row_bytes = 0;
+  if (bias_staged) {
+    const int elt = prm.bias.is_f32 ? 4 : 2;
+    const int g = prm.bias.is_f32 ? lane >> 3 : lane >> 2, piece = prm.bias.is_f32 ? lane & 7 : lane & 3;
+    const int row_in = 8 * (g >> 3) + 4 * (g & 1) + ((g >> 1) & 3);   // the row kept in slot g
+    bias_row_bytes = prm.bias.strides[2] * elt;
+    bias_lane_off = (uint32_t)(row_in * bias_row_bytes + piece * 16);
+    bias_src = (const char*)prm.bias.ptr + (b * prm.bias.strides[0] + h * prm.bias.strides[1] + k0 + wave_s * 32) * elt;   // wave-uniform
+  }
+  auto issue_bias = [&](int qt, int buf) {
+    if (!bias_staged || qt * kBwdTile + kBwdTile > Sq) return;
+    const int rows_per_dma = prm.bias.is_f32 ? 8 : 16, n_dma = prm.bias.is_f32 ? 8 : 4;
+    FO_LDS char* dst = bias_lds + buf * kBiasWaveBytes;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < n_dma) dma16_lane_ptr(bias_src + (int64_t)(qt * kBwdTile + i * rows_per_dma) * bias_row_bytes + bias_lane_off, dst + i * 1024);
+  };
   auto issue = [&](int qt, int buf) {
+    if constexpr (BIAS) issue_bias(qt, buf);
     if (qt * kBwdTile + kBwdTile <= Sq && qlo.ok && glo.ok) {
       copy_tile64_inside<T, D>(qbase, prm.qs[2], qt * kBwdTile, qlo, smem + buf * TILE_BYTES, wave_s);
       copy_tile64_inside<T, D>(gbase, prm.dos[2], qt * kBwdTile, glo, smem + (2 + buf) * TILE_BYTES, wave_s);
@@ -435,6 +492,32 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
       f32x16 sacc, dpacc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sacc[r] = 0.0f; dpacc[r] = 0.0f; }
+      // the staged bias of this block's 16 registers, read ahead of the MFMAs below (read where it is used, each
+      // value is waited for on its own): row 32*qb + 8*j + 4*hh + u of the tile sits in copy instruction 4*qb + j
+      // (fp32) or 2*qb + j/2 (operand type)
+      float bias_reg[BIAS ? 16 : 1];
+      const bool bias_from_lds = BIAS && bias_staged && q0t + kBwdTile <= Sq;
+      if constexpr (BIAS) {
+        if (bias_from_lds) {
+          FO_LDS const char* bias_t = bias_lds + buf * kBiasWaveBytes + (prm.bias.is_f32 ? hh * 128 + l32 * 4 : hh * 64 + l32 * 2);
+          // (one decision on the bias type around all 16 reads: decided per element, every read gets its own branch
+          // and its own wait)
+          if (prm.bias.is_f32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+              for (int u = 0; u < 4; ++u) bias_reg[4 * j + u] = *(FO_LDS const float*)(bias_t + (4 * qb + j) * 1024 + u * 256);
+          } else {
+            T raw[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+              for (int u = 0; u < 4; ++u) raw[4 * j + u] = *(FO_LDS const T*)(bias_t + (2 * qb + (j >> 1)) * 1024 + (j & 1) * 512 + u * 128);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bias_reg[r] = (float)raw[r];
+          }
+        }
+      }
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         sacc = Ops<T>::mfma(row_frag<T, D>(qtile, qb, ks, l32, hh), kf[ks], sacc);      // S = Q K^T
@@ -449,7 +532,9 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
       const uint32_t drop_base = DROP ? prm.drop.offset + ((uint32_t)bh * (uint32_t)Sq + (uint32_t)(q0t + 32 * qb + 4 * hh)) * (uint32_t)Sk + (uint32_t)key : 0u;
       // bias column of this lane's key; queries past the end re-read the last one
       const int64_t bias_col = BIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] + krow : 0;
-      auto softmax_grad = [&](auto masked) {
+      // where the bias comes from: 0 global memory, element by element; 1 the lane's own value; 2 the staged tile
+      auto softmax_grad = [&](auto masked, auto bias_mode) {
+      constexpr int BM = decltype(bias_mode)::value;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 l4 = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * j + 4 * hh);
@@ -459,10 +544,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
           const int r = 4 * j + u;
           const bool dead = decltype(masked)::value && ((u + 8 * j) < lim || (u + 8 * j) >= lim_end);
           float shift = -l4[u] * kLog2e;
-          if constexpr (BIAS) {
+          if constexpr (BIAS && BM == 0) {
             const int qi = min(q0t + 32 * qb + 4 * hh + u + 8 * j, Sq - 1);
             shift = __builtin_fmaf(load_bias<T>(prm.bias, bias_col + (int64_t)qi * prm.bias.strides[2]), kLog2e, shift);
           }
+          if constexpr (BIAS && BM == 1) shift += bias_lane;
+          if constexpr (BIAS && BM == 2) shift = __builtin_fmaf(bias_reg[r], kLog2e, shift);
           const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], c, shift));
           float pd = p, dp = dpacc[r];
           if constexpr (DROP) {
@@ -475,8 +562,19 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
         }
       }
       };
-      if (q0t + 32 * qb + 32 > Sq || (CAUSAL && k0w + 31 > q0t + 32 * qb)) softmax_grad(std::true_type{});
-      else softmax_grad(std::false_type{});
+      const bool needs_mask = q0t + 32 * qb + 32 > Sq || (CAUSAL && k0w + 31 > q0t + 32 * qb);
+      typedef std::integral_constant<int, 0> BM0;
+      typedef std::integral_constant<int, 1> BM1;
+      typedef std::integral_constant<int, 2> BM2;
+      if constexpr (!BIAS) {
+        if (needs_mask) softmax_grad(std::true_type{}, BM0{}); else softmax_grad(std::false_type{}, BM0{});
+      } else if (bias_per_key) {
+        if (needs_mask) softmax_grad(std::true_type{}, BM1{}); else softmax_grad(std::false_type{}, BM1{});
+      } else if (bias_from_lds) {
+        if (needs_mask) softmax_grad(std::true_type{}, BM2{}); else softmax_grad(std::false_type{}, BM2{});
+      } else {
+        if (needs_mask) softmax_grad(std::true_type{}, BM0{}); else softmax_grad(std::false_type{}, BM0{});
+      }
       // dV^T += dO^T P and dK^T += Q^T dS : two 16-query steps x DBLK d-blocks
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -764,7 +862,7 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   const int64_t g_dkdv = ((p.Sk + kBwdRows - 1) / kBwdRows) * n_bh;
   if (g_delta > 0x7FFFFFFFll || g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
   const size_t lds_dq = 4 * (size_t)kBwdTile * D * 2;
-  const size_t lds_dkdv = lds_dq + 4 * kBwdTile * sizeof(float);
+  const size_t lds_dkdv = lds_dq + 4 * kBwdTile * sizeof(float) + (BIAS ? kBwdWaves * 2 * kBwdTile * 32 * 4 : 0);   // + bias tiles
   static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
   static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS>,
@@ -842,7 +940,13 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   p.bias.ptr = bias;
   for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
   p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
-  p.bias.dma_ok = 0;   // (the backward kernels read the bias element by element)
+  {
+    const uintptr_t elt = p.bias.is_f32 ? 4 : 2;
+    // (dK/dV kernel: tiles of the bias are copied into LDS in 16-byte pieces)
+    p.bias.dma_ok = bias && p.bias.strides[2] != 0 && ((uintptr_t)bias % 16) == 0 && (p.bias.strides[0] * elt) % 16 == 0 &&
+                    (p.bias.strides[1] * elt) % 16 == 0 && (p.bias.strides[2] * elt) % 16 == 0;
+    p.bias.vec_ok = bias && ((uintptr_t)bias % (4 * elt)) == 0 && p.bias.strides[0] % 4 == 0 && p.bias.strides[1] % 4 == 0 && p.bias.strides[2] % 4 == 0;
+  }
 #define FO_BWD2(T, DD, BI) (drop ? (c ? launch_bwd<T, DD, true, true, BI>(p, s) : launch_bwd<T, DD, false, true, BI>(p, s)) \
                                  : (c ? launch_bwd<T, DD, true, false, BI>(p, s) : launch_bwd<T, DD, false, false, BI>(p, s)))
 #define FO_BWD(T, DD) (bias ? FO_BWD2(T, DD, true) : FO_BWD2(T, DD, false))

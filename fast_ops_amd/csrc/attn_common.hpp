@@ -79,11 +79,20 @@ struct BiasParams {
   const void* ptr;
   int64_t strides[3];
   int is_f32;
-  int dma_ok;   // base and the three strides are multiples of 16 bytes: tiles may be copied with 16-byte pieces
+  int dma_ok;   // forward: base and the three strides are multiples of 16 bytes, tiles may be copied with 16-byte pieces
+  int vec_ok;   // backward: base and the three strides are multiples of 4 elements, 4 keys may be read with one load
 };
 template <typename T>
 __device__ __forceinline__ float load_bias(const BiasParams& bp, int64_t at) {
   return bp.is_f32 ? ((const float*)bp.ptr)[at] : (float)((const T*)bp.ptr)[at];
+}
+// four consecutive elements of type E (float or the operand type) from an address that is a multiple of 4 elements
+template <typename E>
+__device__ __forceinline__ void load_bias4(const E* at, float* out) {
+  typedef __attribute__((ext_vector_type(4))) E e4;
+  const e4 t = *(const e4*)at;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) out[u] = (float)t[u];
 }
 
 // the same with 4 bytes per lane (LDS receives 256 bytes)

@@ -1132,6 +1132,7 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   p.bias.ptr = bias;
   for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
   p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
+  p.bias.vec_ok = 0;
   {
     const int64_t elt = p.bias.is_f32 ? 4 : 2;
     // (a bias that is the same for every query - query stride 0 - is one row per tile: per-element loads of it are
