@@ -224,7 +224,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   constexpr int KSTEPS = D / 16;
   constexpr int DBLK = D / 32;
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
-  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // K0 | K1 | V0 | V1
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // K0 | K1 | V0 | V1 | bias of the tile's 64 keys, two buffers (BIAS)
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
@@ -243,7 +243,25 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   TileLaneOffsets<T, D> klo, vlo;
   klo.init(prm.ks[2], wave_s, lane);
   vlo.init(prm.vs[2], wave_s, lane);
+  // A bias that is the same for every query (query stride 0) is 64 values per key tile, the same for all lanes: wave 0
+  // copies them into LDS with the tile (4 bytes per lane: one key in fp32, two in the operand type), and every lane
+  // reads its registers' keys from there. (Loaded from global memory where they are used, the compiler waits for
+  // them together with the tile copies in flight.) Keys past the end re-read the last ones and are masked below.
+  FO_LDS char* bias_keys = smem + 4 * TILE_BYTES;
+  bool bias_keys_staged = false;
+  const char* bias_keys_src = nullptr;
+  if constexpr (BIAS) {
+    const int64_t at = b * prm.bias.strides[0] + h * prm.bias.strides[1];
+    bias_keys_src = (const char*)prm.bias.ptr + at * (prm.bias.is_f32 ? 4 : 2);
+    bias_keys_staged = prm.bias.strides[2] == 0 && ((uintptr_t)bias_keys_src % 4) == 0 && (prm.bias.is_f32 || Sk % 2 == 0);   // (pairs of keys: an even count)
+  }
   auto issue = [&](int tile, int buf) {
+    if constexpr (BIAS) {
+      if (bias_keys_staged && wave_s == 0) {
+        if (prm.bias.is_f32) dma4_lane_ptr(bias_keys_src + (int64_t)min(tile * kBwdTile + lane, Sk - 1) * 4, bias_keys + buf * 256);
+        else if (lane < 32) dma4_lane_ptr(bias_keys_src + (int64_t)min(tile * kBwdTile + 2 * lane, Sk - 2) * 2, bias_keys + buf * 256);
+      }
+    }
     if (tile * kBwdTile + kBwdTile <= Sk && klo.ok && vlo.ok) {
       copy_tile64_inside<T, D>(kbase, prm.ks[2], tile * kBwdTile, klo, smem + buf * TILE_BYTES, wave_s);
       copy_tile64_inside<T, D>(vbase, prm.vs[2], tile * kBwdTile, vlo, smem + (2 + buf) * TILE_BYTES, wave_s);
@@ -315,36 +333,66 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
         const int key_base = key0 + 32 * kb + 4 * hh;
         int lim = key_base - Sk + 1;
         if (CAUSAL) lim = max(lim, key_base - (q0w + l32));
-        // the bias of this lane's 16 keys: four loads of four consecutive keys when the tile is complete and the
-        // bias is laid out for it, else key by key (every lane reads its own row: an instruction touches 32 cache
-        // lines either way, so fewer instructions is what counts)
-        float bv[BIAS ? 16 : 1];
-        if constexpr (BIAS) {
-          if (prm.bias.vec_ok && key0 + kBwdTile <= Sk) {
-            if (prm.bias.is_f32) {
+        // registers 4*j .. 4*j + 3 (four consecutive keys), given their bias
+        auto four = [&](int j, const float* b4) {
 #pragma unroll
-              for (int j = 0; j < 4; ++j) load_bias4<float>((const float*)prm.bias.ptr + bias_row + key_base + 8 * j, bv + 4 * j);
-            } else {
+          for (int u = 0; u < 4; ++u) {
+            const int r = 4 * j + u;
+            const bool dead = decltype(masked)::value && lim > -(u + 8 * j);
+            float shift = -lse2;
+            if constexpr (BIAS) shift = __builtin_fmaf(b4[u], kLog2e, -lse2);
+            const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, shift));
+            float dp = dpacc[kb][r];
+            if constexpr (DROP) {
+              const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + u + 8 * j);
+              dp = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? dp * prm.drop.keep_scale : 0.0f;
+            }
+            dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp - delta));
+          }
+        };
+        // The bias of four keys at a time (few values in flight: this kernel has no registers to spare). From the
+        // per-key values staged in LDS; else with one load of four consecutive keys when the tile is complete and the
+        // bias is laid out for it; else key by key. Every lane reads its own row, so a load instruction touches 32
+        // cache lines either way, and fewer instructions is what counts. The bias type is decided around the loops.
+        float b4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (!BIAS) {
 #pragma unroll
-              for (int j = 0; j < 4; ++j) load_bias4<T>((const T*)prm.bias.ptr + bias_row + key_base + 8 * j, bv + 4 * j);
+          for (int j = 0; j < 4; ++j) four(j, b4);
+        } else if (bias_keys_staged) {
+          FO_LDS const char* bk = bias_keys + buf * 256;
+          if (prm.bias.is_f32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const f32x4 t4 = *(FO_LDS const f32x4*)(bk + (32 * kb + 4 * hh + 8 * j) * 4);
+#pragma unroll
+              for (int u = 0; u < 4; ++u) b4[u] = t4[u];
+              four(j, b4);
             }
           } else {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) bv[r] = load_bias<T>(prm.bias, bias_row + min(key_base + (r & 3) + 8 * (r >> 2), Sk - 1));
-          }
-        }
+            for (int j = 0; j < 4; ++j) {
+              typedef __attribute__((ext_vector_type(4))) T vec4;
+              const vec4 t4 = *(FO_LDS const vec4*)(bk + (32 * kb + 4 * hh + 8 * j) * 2);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const bool dead = decltype(masked)::value && lim > -((r & 3) + 8 * (r >> 2));
-          float shift = -lse2;
-          if constexpr (BIAS) shift = __builtin_fmaf(bv[r], kLog2e, -lse2);
-          const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], c, shift));
-          float dp = dpacc[kb][r];
-          if constexpr (DROP) {
-            const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2));
-            dp = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? dp * prm.drop.keep_scale : 0.0f;
+              for (int u = 0; u < 4; ++u) b4[u] = (float)t4[u];
+              four(j, b4);
+            }
           }
-          dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp - delta));
+        } else if (prm.bias.vec_ok && key0 + kBwdTile <= Sk) {
+          if (prm.bias.is_f32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { load_bias4<float>((const float*)prm.bias.ptr + bias_row + key_base + 8 * j, b4); four(j, b4); }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { load_bias4<T>((const T*)prm.bias.ptr + bias_row + key_base + 8 * j, b4); four(j, b4); }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) b4[u] = load_bias<T>(prm.bias, bias_row + min(key_base + u + 8 * j, Sk - 1));
+            four(j, b4);
+          }
         }
       }
     };
@@ -861,8 +909,9 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   const int64_t g_dq = ((p.Sq + kBwdRows - 1) / kBwdRows) * n_bh;
   const int64_t g_dkdv = ((p.Sk + kBwdRows - 1) / kBwdRows) * n_bh;
   if (g_delta > 0x7FFFFFFFll || g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
-  const size_t lds_dq = 4 * (size_t)kBwdTile * D * 2;
-  const size_t lds_dkdv = lds_dq + 4 * kBwdTile * sizeof(float) + (BIAS ? kBwdWaves * 2 * kBwdTile * 32 * 4 : 0);   // + bias tiles
+  const size_t lds_tiles = 4 * (size_t)kBwdTile * D * 2;
+  const size_t lds_dq = lds_tiles + (BIAS ? 512 : 0);   // + the per-key bias of two tiles
+  const size_t lds_dkdv = lds_tiles + 4 * kBwdTile * sizeof(float) + (BIAS ? kBwdWaves * 2 * kBwdTile * 32 * 4 : 0);   // + bias tiles
   static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
   static const hipError_t a2 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS>,

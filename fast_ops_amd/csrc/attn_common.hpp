@@ -80,7 +80,7 @@ struct BiasParams {
   int64_t strides[3];
   int is_f32;
   int dma_ok;   // forward: base and the three strides are multiples of 16 bytes, tiles may be copied with 16-byte pieces
-  int vec_ok;   // backward: base and the three strides are multiples of 4 elements, 4 keys may be read with one load
+  int vec_ok;   // base and the three strides are multiples of 4 elements: 4 consecutive keys may be read with one load
 };
 template <typename T>
 __device__ __forceinline__ float load_bias(const BiasParams& bp, int64_t at) {

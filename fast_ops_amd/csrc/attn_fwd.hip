@@ -285,33 +285,61 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
       if (prm.bias.dma_ok && key0 + kBN <= Sk) {
         // from the tile copied into LDS: register r = 4 j + u of block kb is key 32 kb + 8 j + 4 hh + u of row l32
         FO_LDS const char* bt = bias_lds + buf * kWaves * kBiasWaveBytes;
+        // (the bias type is decided once around the unrolled loops: decided per element, every read gets a branch)
+        if (prm.bias.is_f32) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+          for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            f32x4 bv;
-            if (prm.bias.is_f32) {
-              bv = *(FO_LDS const f32x4*)(bt + l32 * 256 + (((8 * kb + 2 * j + hh) ^ (l32 & 15)) * 16));
-            } else {
+            for (int j = 0; j < 4; ++j) {
+              const f32x4 bv = *(FO_LDS const f32x4*)(bt + l32 * 256 + (((8 * kb + 2 * j + hh) ^ (l32 & 15)) * 16));
+#pragma unroll
+              for (int u = 0; u < 4; ++u)
+                sacc[kb][4 * j + u] = __builtin_fmaf(sacc[kb][4 * j + u], prm.scale_log2e, bv[u] * 1.4426950408889634f);
+            }
+        } else {
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
               typedef __attribute__((ext_vector_type(4))) T vec4;
               const vec4 h4 = *(FO_LDS const vec4*)(bt + l32 * 128 + (((4 * kb + j) ^ (l32 & 7)) * 16) + hh * 8);
 #pragma unroll
-              for (int u = 0; u < 4; ++u) bv[u] = (float)h4[u];
+              for (int u = 0; u < 4; ++u)
+                sacc[kb][4 * j + u] = __builtin_fmaf(sacc[kb][4 * j + u], prm.scale_log2e, (float)h4[u] * 1.4426950408889634f);
             }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-              sacc[kb][4 * j + u] = __builtin_fmaf(sacc[kb][4 * j + u], prm.scale_log2e, bv[u] * 1.4426950408889634f);
-          }
+        }
       } else {
-        // per-element loads; rows and keys past the end re-read the last ones
+        // loads from global memory: four consecutive keys per load when the tile is complete and the bias is laid out
+        // for it, else key by key; rows and keys past the end re-read the last ones
         const int64_t brow = b * prm.bias.strides[0] + h * prm.bias.strides[1] + (int64_t)min(q0w + l32, Sq - 1) * prm.bias.strides[2];
+        float bv[2][16];
+        if (prm.bias.vec_ok && key0 + kBN <= Sk) {
+          if (prm.bias.is_f32) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) load_bias4<float>((const float*)prm.bias.ptr + brow + key0 + 32 * kb + 4 * hh + 8 * j, bv[kb] + 4 * j);
+          } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) load_bias4<T>((const T*)prm.bias.ptr + brow + key0 + 32 * kb + 4 * hh + 8 * j, bv[kb] + 4 * j);
+          }
+        } else if (prm.bias.is_f32) {
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bv[kb][r] = ((const float*)prm.bias.ptr)[brow + min(key0 + 32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2), Sk - 1)];
+        } else {
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bv[kb][r] = (float)((const T*)prm.bias.ptr)[brow + min(key0 + 32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2), Sk - 1)];
+        }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = min(key0 + 32 * kb + 4 * hh + (r & 3) + 8 * (r >> 2), Sk - 1);
-            sacc[kb][r] = __builtin_fmaf(sacc[kb][r], prm.scale_log2e, load_bias<T>(prm.bias, brow + key) * 1.4426950408889634f);
-          }
+          for (int r = 0; r < 16; ++r) sacc[kb][r] = __builtin_fmaf(sacc[kb][r], prm.scale_log2e, bv[kb][r] * 1.4426950408889634f);
       }
     }
 
@@ -1132,9 +1160,9 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   p.bias.ptr = bias;
   for (int i = 0; i < 3; ++i) p.bias.strides[i] = bias ? bias_strides[i] : 0;
   p.bias.is_f32 = bias_dtype == FO_DTYPE_F32;
-  p.bias.vec_ok = 0;
   {
     const int64_t elt = p.bias.is_f32 ? 4 : 2;
+    p.bias.vec_ok = bias && ((uintptr_t)bias % (4 * elt)) == 0 && p.bias.strides[0] % 4 == 0 && p.bias.strides[1] % 4 == 0 && p.bias.strides[2] % 4 == 0;
     // (a bias that is the same for every query - query stride 0 - is one row per tile: per-element loads of it are
     // broadcasts, and the kernel keeps its two workgroups per CU without the LDS for bias tiles)
     p.bias.dma_ok = bias && p.bias.strides[2] != 0 && ((uintptr_t)bias % 16) == 0 && (p.bias.strides[0] * elt) % 16 == 0 &&
