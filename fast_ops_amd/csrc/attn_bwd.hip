@@ -118,7 +118,7 @@ __device__ __forceinline__ void acc_fence(f32x16 (&acc)[N]) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-// delta[b, h, q] = sum_d dO * O   (flash_attention_triton.py:273-315). Eight lanes per row.
+// delta[b, h, q] = sum_d dO * O   (flash_attention_triton.py:273-315), stored negated. Eight lanes per row.
 template <typename T, int D>
 __global__ void __launch_bounds__(256) attn_bwd_delta_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(256) attn_bwd_delta_kernel(const AttnBwdParams
   acc += __shfl_xor(acc, 1);
   acc += __shfl_xor(acc, 2);
   acc += __shfl_xor(acc, 4);
-  if (row < n_rows && j == 0) prm.delta[row] = acc;
+  if (row < n_rows && j == 0) prm.delta[row] = -acc;   // negated: the kernels below add it to dP, or start dP from it
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -282,7 +282,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     for (int ks = 0; ks < KSTEPS; ++ks) { qf[ks] = *(const vec8*)(qp + 16 * ks); gf[ks] = *(const vec8*)(gp + 16 * ks); }
   }
   const float lse2 = prm.lse[(int64_t)bh * Sq + qrow] * kLog2e;
-  const float delta = prm.delta[(int64_t)bh * Sq + qrow];
+  const float delta = prm.delta[(int64_t)bh * Sq + qrow];   // -delta
   // (consumed here so that the compiler waits for these loads before the loop: a vmcnt wait inside the loop would
   // also wait for the tile copies in flight, which it does not see)
 #pragma unroll
@@ -347,7 +347,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
               const uint32_t idx = drop_row + (uint32_t)(32 * kb + 4 * hh + u + 8 * j);
               dp = dropout_keep(idx, prm.drop.seed, prm.drop.threshold) ? dp * prm.drop.keep_scale : 0.0f;
             }
-            dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp - delta));
+            dsf[kb * 2 + (r >> 3)][r & 7] = (T)(p * (dp + delta));
           }
         };
         // The bias of four keys at a time (few values in flight: this kernel has no registers to spare). From the
@@ -606,7 +606,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
             dp = keep ? dp * prm.drop.keep_scale : 0.0f;
           }
           pf[r >> 3][r & 7] = (T)pd;
-          dsf[r >> 3][r & 7] = (T)(p * (dp - d4[u]));   // softmax_scale is applied to the finished dK
+          dsf[r >> 3][r & 7] = (T)(p * (dp + d4[u]));   // (d4 = -delta) softmax_scale is applied to the finished dK
         }
       }
       };
@@ -768,7 +768,11 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   static_assert((4 * NMF) % kFragAhead == 0, "the fragment ring runs on across tiles");
   vec8 fr[kFragAhead];         // A operands, fetched kFragAhead micro-groups ahead of their MFMA
   f32x16 sacc[2], dpacc[2];
-  vec8 pf[2][2], dsf[2][2];
+  // P and dS as B operands: pairs of 16-bit values, kept as 32-bit words so that a finished pair can be pinned
+  typedef __attribute__((ext_vector_type(4))) int i32x4;
+  typedef __attribute__((ext_vector_type(2))) T vec2;
+  i32x4 pf[2][2], dsf[2][2];
+  float p_even[2] = {0.0f, 0.0f}, ds_even[2] = {0.0f, 0.0f};
 
   auto tile_body = [&](int j, auto masked) {
     const int buf = (j - qt0) % NBUF, nbuf = (buf + 1) % NBUF;
@@ -793,14 +797,24 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     };
     FO_LDS const float* lse_t = rowvals + buf * kBwdTile;
     FO_LDS const float* del_t = rowvals + (NBUF + buf) * kBwdTile;
-    f32x4 lv[2], dv[2];        // LSE and delta of four query rows, fetched one vector ahead
+    f32x4 lv[2];               // LSE of four query rows, fetched one vector ahead
+    // dP = dO V^T - delta comes out of the MFMAs: the accumulator of a block's dP starts from -delta of its 16 rows,
+    // read from LDS straight into the accumulator registers while they are idle (block 1: during phase 1; block 0 of
+    // the next tile: during phase 4, after the hand-over made that tile visible)
+    auto start_dp = [&](f32x16& acc, FO_LDS const float* del, int qb) {
+#pragma unroll
+      for (int jv = 0; jv < 4; ++jv) {
+        const f32x4 d4 = *(FO_LDS const f32x4*)(del + 32 * qb + 8 * jv + 4 * hh);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc[4 * jv + u] = d4[u];
+      }
+    };
     // score element r of block qb: register r holds query q0t + 32*qb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2);
     // dead iff key > query or the query is past the end
     auto element = [&](int qb, int r) {
       const int jv = r >> 2, u = r & 3;
       if (u == 0 && jv + 1 < 4) {
         lv[(jv + 1) & 1] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * (jv + 1) + 4 * hh);
-        dv[(jv + 1) & 1] = *(FO_LDS const f32x4*)(del_t + 32 * qb + 8 * (jv + 1) + 4 * hh);
       }
       const int koff = u + 8 * jv;
       bool dead = false;
@@ -810,20 +824,32 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
         dead = koff < lim || koff >= lim_end;
       }
       const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][r], c, -lv[jv & 1][u] * kLog2e));
-      pf[qb][r >> 3][r & 7] = (T)p;
-      dsf[qb][r >> 3][r & 7] = (T)(p * (dpacc[qb][r] - dv[jv & 1][u]));   // softmax_scale is applied to the finished dK
+      const float ds = p * dpacc[qb][r];   // (dP - delta) softmax_scale is applied to the finished dK
+      if (r & 1) {
+        // a finished pair is rounded and pinned to its micro-group: left alone, the compiler moves the multiplication
+        // and the rounding down to the MFMA that reads them, which may not read a register that a VALU instruction
+        // has just written
+        const vec2 p2 = {(T)p_even[qb], (T)p}, ds2 = {(T)ds_even[qb], (T)ds};
+        int pw = __builtin_bit_cast(int, p2), dsw = __builtin_bit_cast(int, ds2);
+        asm volatile("" : "+v"(pw), "+v"(dsw));
+        pf[qb][r >> 3][(r & 7) >> 1] = pw;
+        dsf[qb][r >> 3][(r & 7) >> 1] = dsw;
+      } else {
+        p_even[qb] = p;
+        ds_even[qb] = ds;
+      }
     };
     auto first_rows = [&](int qb) {
       lv[0] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 4 * hh);
-      dv[0] = *(FO_LDS const f32x4*)(del_t + 32 * qb + 4 * hh);
     };
     // ---- phase 1
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = i;
-      if (i & 1) mfma_scores_vgpr<T>(dpacc[0], fr[g % kFragAhead], vf[i >> 1], i == 1); else mfma_scores_vgpr<T>(sacc[0], fr[g % kFragAhead], kf[i >> 1], i == 0);
+      if (i & 1) mfma_scores_vgpr<T>(dpacc[0], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[0], fr[g % kFragAhead], kf[i >> 1], i == 0);
       refill(g);
+      if (i == 0) start_dp(dpacc[1], del_t, 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- phase 2
@@ -831,7 +857,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = NMF + i;
-      if (i & 1) mfma_scores_vgpr<T>(dpacc[1], fr[g % kFragAhead], vf[i >> 1], i == 1); else mfma_scores_vgpr<T>(sacc[1], fr[g % kFragAhead], kf[i >> 1], i == 0);
+      if (i & 1) mfma_scores_vgpr<T>(dpacc[1], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[1], fr[g % kFragAhead], kf[i >> 1], i == 0);
       refill(g);
       if (i == 0) scores_fence(sacc[0], dpacc[0]);
 #pragma unroll
@@ -844,7 +870,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     for (int i = 0; i < NMF; ++i) {
       const int g = 2 * NMF + i;
       const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
-      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], dsf[0][t]); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], pf[0][t]);
+      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, dsf[0][t])); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, pf[0][t]));
       refill(g);
       if (i == 0) scores_fence(sacc[1], dpacc[1]);
 #pragma unroll
@@ -853,12 +879,16 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     }
     if (j + 1 < n_qt) hand_over(j);
     // ---- phase 4
+    // (two wait states: the paths around the hand-over join here, and the check of the generated code, which follows
+    // no branches, must see that the first MFMA does not read a register written by the VALU instruction before it)
+    asm volatile("s_nop 1");
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = 3 * NMF + i;
       const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
-      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], dsf[1][t]); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], pf[1][t]);
+      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, dsf[1][t])); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, pf[1][t]));
       refill(g);
+      if (i == 0) start_dp(dpacc[0], rowvals + (NBUF + nbuf) * kBwdTile, 0);   // (after the last tile: read, unused)
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -877,6 +907,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     for (int ks = 0; ks < (kFragAhead + 1) / 2; ++ks) rq0[ks] = row_off[ks] + (uint32_t)(buf * TILE_BYTES);
 #pragma unroll
     for (int i = 0; i < kFragAhead; ++i) fr[i] = scores_frag(rq0, 0, i);
+    // (dP of the first tile's block 0 starts from -delta, as every later one does at the end of the tile before it)
+#pragma unroll
+    for (int jv = 0; jv < 4; ++jv) {
+      const f32x4 d4 = *(FO_LDS const f32x4*)(rowvals + (NBUF + buf) * kBwdTile + 8 * jv + 4 * hh);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) dpacc[0][4 * jv + u] = d4[u];
+    }
   }
   for (; j < n_qt && needs_mask(j); ++j) tile_body(j, std::true_type{});
   for (; j < n_qt && !needs_mask(j); ++j) tile_body(j, std::false_type{});
