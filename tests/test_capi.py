@@ -150,6 +150,11 @@ def test_tune_hook():
     assert lib.fo_tune_set(b"lion.variant", 3) == 0 and lib.fo_tune_get(b"lion.variant") == 3
     assert lib.fo_tune_set(b"lion.variant", -1) == 0
     assert lib.fo_tune_set(b"no.such.key", 1) == -8
+    # every key the kernels read: default -1 (the library's choice), settable, readable
+    for key in (b"attn.variant", b"attn_bwd.variant", b"attn.order", b"attn_bwd.order"):
+        assert lib.fo_tune_get(key) == -1
+        assert lib.fo_tune_set(key, 2) == 0 and lib.fo_tune_get(key) == 2
+        assert lib.fo_tune_set(key, -1) == 0 and lib.fo_tune_get(key) == -1
 
 
 def test_python_surfaces_validate_like_the_reference():
