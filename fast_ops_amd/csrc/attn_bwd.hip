@@ -216,6 +216,36 @@ __device__ __forceinline__ typename Ops<T>::vec8 col_frag(FO_LDS const char* til
   return __builtin_bit_cast(typename Ops<T>::vec8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
+// A wave's 32 finished gradient rows (accumulator layout: lane = row l32, registers 4*rg + u = columns
+// 32*db + 8*rg + 4*hh + u) written to memory. Straight from the registers that is 8 bytes per lane to 32 different
+// rows per instruction (4.3 us per workgroup for dK and dV, during which the workgroup's LDS and registers keep the
+// next one waiting); instead the rows are rounded into LDS (`stage`, 32 rows padded by 16 bytes each, this wave's
+// own) and leave as whole 16-byte pieces, 64 lanes covering consecutive rows. Rows from n_rows on are not written.
+template <typename T, int D>
+__device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], float mul, FO_LDS char* stage, T* base, int64_t stride,
+                                                   int row0, int n_rows, int lane) {
+  constexpr int ROW_BYTES = D * 2, OROW = ROW_BYTES + 16, CH = ROW_BYTES / 16;
+  typedef __attribute__((ext_vector_type(4))) T vec4;
+  typedef __attribute__((ext_vector_type(4))) int i32x4;
+  const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      vec4 o4;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) o4[u] = (T)(acc[db][rg * 4 + u] * mul);
+      *(FO_LDS vec4*)(stage + l32 * OROW + (32 * db + 8 * rg + 4 * hh) * 2) = o4;
+    }
+#pragma unroll
+  for (int it = 0; it < 32 * CH / 64; ++it) {
+    const int idx = it * 64 + lane, row = idx / CH, ch = idx % CH;
+    const i32x4 piece = *(FO_LDS const i32x4*)(stage + row * OROW + ch * 16);
+    if (row0 + row < n_rows) *(i32x4*)(base + (int64_t)(row0 + row) * stride + ch * 8) = piece;
+  }
+}
+constexpr int stage_bytes(int D) { return 32 * (D * 2 + 16); }   // per wave and matrix
+
 // ---------------------------------------------------------------------------------------------------------------------
 template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const AttnBwdParams prm) {
@@ -405,6 +435,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
       for (int db = 0; db < DBLK; ++db) acc[db] = Ops<T>::mfma(col_frag<T, D>(kt, t, db, lane), dsf[t], acc[db]);
   }
 
+  // (straight from the registers, 8 bytes per lane: with two workgroups per CU the other one covers the time these
+  // stores take, and staging the rows in LDS as the dK/dV kernels do made this kernel 5-10 % slower)
   const int qi = q0w + l32;
   if (qi < Sq) {
     T* op = (T*)prm.dq + b * prm.dqs[0] + h * prm.dqs[1] + (int64_t)qi * prm.dqs[2];
@@ -634,20 +666,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
     }
   }
 
-  if (key < Sk) {
-    T* kp = (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1] + (int64_t)key * prm.dks[2];
-    T* vp = (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1] + (int64_t)key * prm.dvs[2];
-#pragma unroll
-    for (int db = 0; db < DBLK; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        typedef __attribute__((ext_vector_type(4))) T vec4;
-        vec4 k4, v4;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) { k4[u] = (T)(dkacc[db][rg * 4 + u] * scale); v4[u] = (T)dvacc[db][rg * 4 + u]; }
-        *(vec4*)(kp + 32 * db + 8 * rg + 4 * hh) = k4;
-        *(vec4*)(vp + 32 * db + 8 * rg + 4 * hh) = v4;
-      }
+  // (the tile buffers are free once every wave is past its last tile; dK, then dV, through the wave's own piece of them)
+  __syncthreads();
+  {
+    FO_LDS char* stage = smem + wave_s * stage_bytes(D);
+    const int k0w_s = k0 + wave_s * 32;
+    store_rows_via_lds<T, D>(dkacc, scale, stage, (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1], prm.dks[2], k0w_s, Sk, lane);
+    store_rows_via_lds<T, D>(dvacc, 1.0f, stage, (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1], prm.dvs[2], k0w_s, Sk, lane);
   }
 }
 
@@ -715,17 +740,30 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     if (j + 2 < n_qt) issue(j + 2, (j + 2 - qt0) % NBUF);
   };
 
-  const int key = k0w + l32;
-  const int krow = min(key, Sk - 1);
+  // B operands held for the whole kernel: K^T and V^T fragments of this lane's key. The block's 128 rows of K and of V
+  // come in like tiles - 16-byte pieces straight into LDS, into the buffers of the second and third tile, which are
+  // still free - and each lane takes its row's pieces from there. (Read from global memory row by row, 32 rows per
+  // instruction, this took 4.4 us, a quarter of a workgroup's time at 512 queries.) Rows past the end re-read the
+  // last one, as the masks below expect. The barrier of the first hand-over comes after every wave has its fragments.
   vec8 kf[KSTEPS], vf[KSTEPS];
   {
-    const T* kp = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1] + (int64_t)krow * prm.ks[2] + 8 * hh;
-    const T* vp = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1] + (int64_t)krow * prm.vs[2] + 8 * hh;
+    const T* kbase = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1];
+    const T* vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) { kf[ks] = *(const vec8*)(kp + 16 * ks); vf[ks] = *(const vec8*)(vp + 16 * ks); }
+    for (int half = 0; half < 2; ++half) {
+      copy_tile64<T, D>(kbase, prm.ks[2], k0 + 64 * half, Sk, smem + (1 + half) * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(vbase, prm.vs[2], k0 + 64 * half, Sk, smem + (NBUF + 1 + half) * TILE_BYTES, wave_s, lane);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    FO_LDS const char* kt = smem + (1 + (wave_s >> 1)) * TILE_BYTES;
+    FO_LDS const char* vt = smem + (NBUF + 1 + (wave_s >> 1)) * TILE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) { kf[ks] = row_frag<T, D>(kt, wave_s & 1, ks, l32, hh); vf[ks] = row_frag<T, D>(vt, wave_s & 1, ks, l32, hh); }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(kf[ks]), "v"(vf[ks]));
   }
+  const int key = k0w + l32;
   f32x16 dkacc[DBLK], dvacc[DBLK];
 #pragma unroll
   for (int i = 0; i < DBLK; ++i)
@@ -921,20 +959,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 
   acc_fence(dkacc);
   acc_fence(dvacc);
-  if (key < Sk) {
-    T* kp = (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1] + (int64_t)key * prm.dks[2];
-    T* vp = (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1] + (int64_t)key * prm.dvs[2];
-#pragma unroll
-    for (int db = 0; db < DBLK; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        typedef __attribute__((ext_vector_type(4))) T vec4;
-        vec4 k4, v4;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) { k4[u] = (T)(dkacc[db][rg * 4 + u] * scale); v4[u] = (T)dvacc[db][rg * 4 + u]; }
-        *(vec4*)(kp + 32 * db + 8 * rg + 4 * hh) = k4;
-        *(vec4*)(vp + 32 * db + 8 * rg + 4 * hh) = v4;
-      }
+  // (the tile buffers are free once every wave is past its last tile; dK, then dV, through the wave's own piece of them)
+  __syncthreads();
+  {
+    FO_LDS char* stage = smem + wave_s * stage_bytes(D);
+    const int k0w_s = k0 + wave_s * 32;
+    store_rows_via_lds<T, D>(dkacc, scale, stage, (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1], prm.dks[2], k0w_s, Sk, lane);
+    store_rows_via_lds<T, D>(dvacc, 1.0f, stage, (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1], prm.dvs[2], k0w_s, Sk, lane);
   }
 }
 
