@@ -930,6 +930,19 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     }
   }
   mfma_result_fence_v(S[0]);
+  // The reference of the exponentials starts as the row maximum of the first sub-tile (dead keys left out as the step
+  // will mask them: lim as there, sub-tile 0; key 0 is never dead, so the maximum is finite). Started from -inf, the
+  // first step takes the recovery path - maxima, every exponential a second time, 64 accumulator registers rescaled -
+  // once per query block, 1-2 us each time.
+#pragma unroll
+  for (int b2 = 0; b2 < QB; ++b2) {
+    int lim = 4 * hh - Sk + 1;
+    if (CAUSAL) lim = max(lim, 4 * hh - (q0w + 32 * b2 + l32));
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : S[0][b2][r]);
+    m_run[b2] = fmaxf(mloc, half_swap(mloc));
+  }
   step(0, P0{}, Y{}, N{}, Y{}, N{}, -1);
   if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, -1);
   // The steps above may have parked a few registers in scratch memory. Wait here, visibly to the compiler, for any
