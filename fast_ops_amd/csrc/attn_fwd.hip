@@ -913,7 +913,12 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   if (Sk % kBN != 0) j_mask = min(j_mask, n_tiles - 1);
 
   // first tile: fill the pipeline - S(0) on its own, then a step that has nothing to multiply yet
-  if (tile_top(0)) { issue(std::false_type{}, 3); issue(std::true_type{}, 2); }
+  // (The code of the first tile is not the loops' code: it keeps a few registers in scratch memory, and every reload
+  // is waited for with a vmcnt wait that also covers the copies in flight. So all three batches issued above land
+  // before it starts - K(0), K(1) and V(0) have to anyway - and batch 0, K(3) and V(2) into slots nobody has used yet,
+  // goes out after it, in front of the loops.)
+  if (!(DBG & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
   {
     const uint32_t kb0 = k_lane + sub_base(0), kb1 = k_lane + sub_base(1);
 #pragma unroll
@@ -949,6 +954,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0) wait that executes on
   // every iteration and also drains the copies in flight, which it does not see.
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), nothing else
+  last_batch = (DBG & 1) ? 0 : issue_batch(0);
   int j = 1;
   for (; j < min(j_mask, n_w - 1); ++j) {
     const bool sp = tile_top(j);
