@@ -85,7 +85,7 @@ def bench_attention(steps, warmup, cpu_baseline):
         },
         "workload": f"attention fwd B={B} H={H} S={S} D={D} bf16 causal, scale 1/sqrt({D})",
     }
-    # the backward of the same workload (dQ, dK, dV; three launches), reported beside the headline, not part of it
+    # the backward of the same workload (dQ, dK, dV; two launches), reported beside the headline, not part of it
     from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided
 
     go = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev)
@@ -97,7 +97,7 @@ def bench_attention(steps, warmup, cpu_baseline):
         "roofline": {"bound": "mfma", "achieved": bwd_flops / (b_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": bwd_flops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": None,
                      "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "flops_per_launch": bwd_flops},
-        "workload": "attention bwd (delta + dQ + dK/dV kernels) of the same shape, FLOPs by the five-GEMM count",
+        "workload": "attention bwd (dQ + dK/dV kernels) of the same shape, FLOPs by the five-GEMM count",
     }
     # yardstick, not part of the headline: the vendor library's plain bf16 GEMM on the same box with the same kind of
     # data. Under a full-chip MFMA load the clock follows the power drawn, which depends on the operand bits (all-zero

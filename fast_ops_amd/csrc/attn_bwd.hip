@@ -8,13 +8,13 @@
 // fp32 scores and accumulators; P and dS are rounded to the operand type before the second GEMMs, as the reference
 // does (:515,:562-563).
 //
-// Three launches, no atomics, no scratch beyond the caller's [B, H, Sq] fp32 `delta` buffer:
-//   1. attn_bwd_delta_kernel: delta.
-//   2. attn_bwd_dq_kernel: one workgroup per 128 query rows (4 waves x 32), walks the key tiles like the forward
+// Two launches, no atomics, no scratch beyond the caller's [B, H, Sq] fp32 `delta` buffer:
+//   1. attn_bwd_dq_kernel: one workgroup per 128 query rows (4 waves x 32), walks the key tiles like the forward
 //      kernel. Scores are computed transposed, S^T = K Q^T and dP^T = V dO^T (A operands = K / V rows from LDS, B
 //      operands = Q^T / dO^T held in registers), so a lane owns one query: LSE and delta are per-lane scalars and
 //      dS^T is, as it stands, the B operand of dQ^T = K^T dS^T (A operand via the transposing LDS read of the K tile).
-//   3. attn_bwd_dkdv_kernel: one workgroup per 128 keys (4 waves x 32), walks the query tiles. Here the scores are
+//      It also computes delta (negated) from the dO fragments it holds and the same pieces of O, and stores it.
+//   2. attn_bwd_dkdv_kernel: one workgroup per 128 keys (4 waves x 32), walks the query tiles. Here the scores are
 //      computed untransposed, S = Q K^T and dP = dO V^T (A operands = Q / dO rows from LDS, B operands = K^T / V^T
 //      held in registers), so a lane owns one key and P, dS are the B operands of dV^T = dO^T P and dK^T = Q^T dS
 //      (A operands via the transposing LDS read of the dO and Q tiles); per-row LSE and delta come from LDS.
@@ -118,33 +118,6 @@ __device__ __forceinline__ void acc_fence(f32x16 (&acc)[N]) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-// delta[b, h, q] = sum_d dO * O   (flash_attention_triton.py:273-315), stored negated. Eight lanes per row.
-template <typename T, int D>
-__global__ void __launch_bounds__(256) attn_bwd_delta_kernel(const AttnBwdParams prm) {
-  typedef typename Ops<T>::vec8 vec8;
-  const int64_t row = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);
-  const int j = threadIdx.x & 7;
-  const int64_t n_rows = (int64_t)prm.B * prm.H * prm.Sq;
-  float acc = 0.0f;
-  if (row < n_rows) {
-    const int s = (int)(row % prm.Sq);
-    const int bh = (int)(row / prm.Sq);
-    const int b = bh / prm.H, h = bh % prm.H;
-    const T* op = (const T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)s * prm.os[2];
-    const T* gp = (const T*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + (int64_t)s * prm.dos[2];
-#pragma unroll
-    for (int c = j; c < D / 8; c += 8) {
-      const vec8 ov = *(const vec8*)(op + 8 * c), gv = *(const vec8*)(gp + 8 * c);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc += (float)ov[i] * (float)gv[i];
-    }
-  }
-  acc += __shfl_xor(acc, 1);
-  acc += __shfl_xor(acc, 2);
-  acc += __shfl_xor(acc, 4);
-  if (row < n_rows && j == 0) prm.delta[row] = -acc;   // negated: the kernels below add it to dP, or start dP from it
-}
-
 // ---------------------------------------------------------------------------------------------------------------------
 // Copy of a 64-row tile (rows row0 .. row0+63 of a [S, D] matrix with row stride `stride`) into LDS by the whole
 // workgroup: per wave D/32 direct-to-LDS instructions. Each instruction fills 1 KiB of LDS with the 64 lanes' pieces
@@ -312,7 +285,21 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     for (int ks = 0; ks < KSTEPS; ++ks) { qf[ks] = *(const vec8*)(qp + 16 * ks); gf[ks] = *(const vec8*)(gp + 16 * ks); }
   }
   const float lse2 = prm.lse[(int64_t)bh * Sq + qrow] * kLog2e;
-  const float delta = prm.delta[(int64_t)bh * Sq + qrow];   // -delta
+  // delta_i = sum_d dO_id O_id (flash_attention_triton.py:273-315), negated: this lane holds half of its row's dO
+  // already, so it reads the same pieces of O, and the two halves of the wave add up. Stored for the dK/dV kernel,
+  // which runs after this one (a pass of its own over O and dO would be a launch more: 5 of 83 us at B=8 H=12 S=1024).
+  float delta = 0.0f;
+  {
+    const T* op = (const T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)qrow * prm.os[2] + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const vec8 ov = *(const vec8*)(op + 16 * ks);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) delta -= (float)ov[e] * (float)gf[ks][e];
+    }
+    delta += half_swap(delta);
+    if (hh == 0 && q0w + l32 < Sq) prm.delta[(int64_t)bh * Sq + q0w + l32] = delta;
+  }
   // (consumed here so that the compiler waits for these loads before the loop: a vmcnt wait inside the loop would
   // also wait for the tile copies in flight, which it does not see)
 #pragma unroll
@@ -971,12 +958,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 
 template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
 static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
-  const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
   const int64_t n_bh = (int64_t)p.B * p.H;
-  const int64_t g_delta = (n_rows + 31) / 32;
   const int64_t g_dq = ((p.Sq + kBwdRows - 1) / kBwdRows) * n_bh;
   const int64_t g_dkdv = ((p.Sk + kBwdRows - 1) / kBwdRows) * n_bh;
-  if (g_delta > 0x7FFFFFFFll || g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
+  if (g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
   const size_t lds_tiles = 4 * (size_t)kBwdTile * D * 2;
   const size_t lds_dq = lds_tiles + (BIAS ? 512 : 0);   // + the per-key bias of two tiles
   const size_t lds_dkdv = lds_tiles + 4 * kBwdTile * sizeof(float) + (BIAS ? kBwdWaves * 2 * kBwdTile * 32 * 4 : 0);   // + bias tiles
@@ -1000,7 +985,7 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
     if (group <= 0 || group > n_bh) group = n_bh;
     q.head_group = (int)group;
   }
-  attn_bwd_delta_kernel<T, D><<<(unsigned)g_delta, 256, 0, s>>>(q);
+  // (delta is computed by the dQ kernel, which the dK/dV kernel follows)
   attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(q);
   // attn_bwd.variant 0 selects the plain dK/dV kernel everywhere (tests compare the two)
   if (!DROP && !BIAS && g_attn_bwd_variant != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(q);

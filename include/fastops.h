@@ -91,7 +91,7 @@ int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
  *   strides_host        eight pointers to three element strides each (batch, head, sequence; head_dim stride 1), in
  *                       the order q, k, v, o, d_o, dq, dk, dv. Only the inputs may repeat a batch or head (stride 0).
  * Same requirements as fo_attn_fwd (D in {64, 128}, 16-byte aligned pointers and rows, scale finite and > 0).
- * Three launches on `stream`; no atomics, results are deterministic.
+ * Two launches on `stream`; no atomics, results are deterministic.
  */
 int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                 float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
