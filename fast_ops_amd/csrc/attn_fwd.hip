@@ -739,7 +739,9 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // m = -inf); only then (rarely) the step's P is recomputed from the still intact scores against the true maximum,
   // and O and l are rescaled. The result is that of the exact recurrence (flash_attention_triton.py:200-213,241-243)
   // up to rounding.
-  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop, int dma_tile) {
+  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop, int dma_tile, auto... no_recovery) {
+    // (an extra argument: the caller knows that no P of this step can be large, and the recovery path is left out)
+    constexpr bool CAN_RECOVER = sizeof...(no_recovery) == 0;
     // inside the loops the MFMAs go without wait states in front unless the build asked for them (see above)
     typedef AsmMfma<T, !(decltype(in_loop)::value && !FO_MFMA_NOPS)> Mfma;
     constexpr int P = decltype(parity)::value;
@@ -847,7 +849,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     bool redo = false;
 #pragma unroll
     for (int b2 = 0; b2 < QB; ++b2) redo = redo || !(psum[b2] <= kLargeRowSum);
-    if (__builtin_amdgcn_ballot_w64(redo) != 0 && !(DBG & 2)) {
+    if (CAN_RECOVER && __builtin_amdgcn_ballot_w64(redo) != 0 && !(DBG & 2)) {
       // rare: true row maxima of this sub-tile, new references, P and row sums again, O and l rescaled
 #pragma unroll
       for (int d = 0; d < DBLK; ++d) mfma_result_fence_a(oacc[d]);
@@ -948,7 +950,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : S[0][b2][r]);
     m_run[b2] = fmaxf(mloc, half_swap(mloc));
   }
-  step(0, P0{}, Y{}, N{}, Y{}, N{}, -1);
+  step(0, P0{}, Y{}, N{}, Y{}, N{}, -1, N{});   // (its reference is its own row maximum: every P <= 1)
   if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, -1);
   // The steps above may have parked a few registers in scratch memory. Wait here, visibly to the compiler, for any
   // reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0) wait that executes on
