@@ -576,6 +576,20 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   }
   const int b = bh / prm.H, h = bh % prm.H;
   const int n_pass = (CAUSAL && prm.n_qblk - 1 - item != item) ? 2 : 1;
+  // Q^T fragments (B operand of S^T = K Q^T), QB blocks of 32 query rows, of the query block a pass works on. The
+  // second pass's are fetched when the first pass has computed its last scores, so that they arrive while it
+  // normalises and writes its O.
+  i32x4 qf[QB][KSTEPS];
+  auto load_q = [&](int for_qblk) {
+    const T* qb_base = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const int qrow = min(for_qblk * kWideBM + wave_s * 32 * QB + 32 * qb + l32, prm.Sq - 1);
+      const T* qp = qb_base + (int64_t)qrow * prm.qs[2] + 8 * hh;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) qf[qb][ks] = *(const i32x4*)(qp + 16 * ks);
+    }
+  };
   for (int pass = 0; pass < n_pass; ++pass) {
   const int qblk = CAUSAL ? (pass == 0 ? prm.n_qblk - 1 - item : item) : item;
   if (pass > 0) {
@@ -586,7 +600,6 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   const int q0 = qblk * kWideBM;
   const int q0w = q0 + wave_s * 32 * QB;
   const int Sq = prm.Sq, Sk = prm.Sk;
-  const T* __restrict__ qbase = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
   const T* __restrict__ kbase = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1];
   const T* __restrict__ vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
 
@@ -679,15 +692,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   issue_batch(-2);
   int last_batch = issue_batch(-1);
 
-  // ---- Q^T fragments (B operand of S^T = K Q^T), QB blocks of 32 query rows
-  i32x4 qf[QB][KSTEPS];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    const int qrow = min(q0w + 32 * qb + l32, Sq - 1);
-    const T* qp = qbase + (int64_t)qrow * prm.qs[2] + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[qb][ks] = *(const i32x4*)(qp + 16 * ks);
-  }
+  if (pass == 0) load_q(qblk);
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
@@ -915,10 +920,10 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   if (Sk % kBN != 0) j_mask = min(j_mask, n_tiles - 1);
 
   // first tile: fill the pipeline - S(0) on its own, then a step that has nothing to multiply yet
-  // (The code of the first tile is not the loops' code: it keeps a few registers in scratch memory, and every reload
-  // is waited for with a vmcnt wait that also covers the copies in flight. So all three batches issued above land
-  // before it starts - K(0), K(1) and V(0) have to anyway - and batch 0, K(3) and V(2) into slots nobody has used yet,
-  // goes out after it, in front of the loops.)
+  // (The code of the first tile is not the loops' code: whenever the compiler parks registers in scratch memory there,
+  // every reload is waited for with a vmcnt wait that also covers the copies in flight. So all three batches issued
+  // above land before it starts - K(0), K(1) and V(0) have to anyway - and batch 0, K(3) and V(2) into slots nobody
+  // has used yet, goes out after it, in front of the loops.)
   if (!(DBG & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
   {
@@ -952,9 +957,9 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   }
   step(0, P0{}, Y{}, N{}, Y{}, N{}, -1, N{});   // (its reference is its own row maximum: every P <= 1)
   if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, -1);
-  // The steps above may have parked a few registers in scratch memory. Wait here, visibly to the compiler, for any
-  // reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0) wait that executes on
-  // every iteration and also drains the copies in flight, which it does not see.
+  // Should the steps above have parked registers in scratch memory (they do not at present), wait here, visibly to
+  // the compiler, for any reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0)
+  // wait that executes on every iteration and also drains the copies in flight, which it does not see.
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), nothing else
   last_batch = (DBG & 1) ? 0 : issue_batch(0);
   int j = 1;
@@ -990,6 +995,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   for (; j < n_tiles; ++j)
     if (tile_top(j)) { issue(std::false_type{}, j + 3); issue(std::true_type{}, j + 2); }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (CAUSAL && pass + 1 < n_pass) load_q(item);   // (the second pass works on query block `item`)
 
   // ---- epilogue: normalise, write O and LSE
 #pragma unroll
