@@ -6,6 +6,11 @@ compiler's hazard recognizer handles for its own MFMA instructions but cannot se
   2. a register written by an 8-pass MFMA (32x32x16 f16/bf16) needs 11 wait states before any other instruction than
      an MFMA touches it.
 
+A third rule concerns the direct-to-LDS copies, which the kernels also issue as inline assembly:
+
+  3. an LDS-DMA instruction (global_load_lds_*, buffer_load_* ... lds) reads M0 and needs 1 wait state after a scalar
+     instruction that wrote M0 (checked by lint_m0_* for every function of a file).
+
 A wait state is one issued instruction (s_nop N counts N+1). For rule 2 time is modelled in wait states; an MFMA is
 taken to issue no earlier than 8 wait states after the previous one (the matrix pipe is busy for its 8 passes), every
 other instruction advances time by one. Control flow is treated conservatively for rule 1 (an MFMA within two
@@ -148,9 +153,64 @@ def lint_file(path: str, name_filter: str) -> List[str]:
     return problems
 
 
+_M0_WRITE = re.compile(r"^s_\w+\s+m0\s*,")
+
+
+def _is_lds_dma(op: str, rest: str) -> bool:
+    if op.startswith("global_load_lds_") or op.startswith("scratch_load_lds_"):
+        return True
+    return op.startswith("buffer_load_") and re.search(r"\blds\b", rest) is not None
+
+
+def lint_m0_function(lines: Iterable[str], name: str) -> List[str]:
+    """Rule 3: no LDS-DMA instruction directly after a scalar write of M0 (or directly after a label, where the
+    predecessor is unknown, if the instruction before the label wrote M0)."""
+    problems: List[str] = []
+    m0_age = 10**9           # wait states since the last scalar write of M0
+    for ln, raw in enumerate(lines, 1):
+        line = raw.split(";")[0].strip()
+        if not line or line.startswith(".") or line.endswith(":"):
+            continue            # labels do not reset the age: a fall-through predecessor counts
+        parts = line.split(None, 1)
+        op, rest = parts[0], (parts[1] if len(parts) > 1 else "")
+        if _is_lds_dma(op, rest) and m0_age < 1:
+            problems.append(f"{name}:{ln}: LDS-DMA reads M0 directly after it was written: {line}")
+        if _M0_WRITE.match(line):
+            m0_age = 0
+            continue
+        states = 1
+        if op == "s_nop":
+            try:
+                states = int(rest.strip(), 0) + 1
+            except ValueError:
+                states = 1
+        m0_age += states
+    return problems
+
+
+def lint_m0_file(path: str) -> List[str]:
+    """Rule 3 over every function of the assembly file."""
+    problems: List[str] = []
+    cur_name, cur_lines = None, []
+    with open(path) as f:
+        for raw in f:
+            s = raw.rstrip("\n")
+            if cur_name is None:
+                head = s.split(";")[0].rstrip()
+                if head.endswith(":") and not head.startswith((".", " ", "\t")):
+                    cur_name, cur_lines = head[:-1], []
+            else:
+                if s.startswith(".Lfunc_end"):
+                    problems += lint_m0_function(cur_lines, cur_name)
+                    cur_name = None
+                else:
+                    cur_lines.append(s)
+    return problems
+
+
 if __name__ == "__main__":
     import sys
-    found = lint_file(sys.argv[1], sys.argv[2] if len(sys.argv) > 2 else "attn_fwd_wide_kernel")
+    found = lint_file(sys.argv[1], sys.argv[2] if len(sys.argv) > 2 else "attn_fwd_wide_kernel") + lint_m0_file(sys.argv[1])
     for p in found[:50]:
         print(p)
     print(f"{len(found)} problem(s)")

@@ -4,7 +4,10 @@ Replaces the reference's import-time JIT builds (fast_ops/flash_attention/flash_
 fast_ops/lion/lion_optimizer.py:15-26) and its setup.py (setup.py:4-18) with one ahead-of-time shared library that
 has a C ABI and no torch or pybind11 dependency. hipcc cross-compiles without a GPU.
 
-Run ``python -m fast_ops_amd.build`` (add ``--force`` to rebuild everything).
+Run ``python -m fast_ops_amd.build`` (add ``--force`` to rebuild everything). ``--ablations`` additionally compiles the
+timing ablations of the attention forward (kernel variants that leave work out and produce wrong results by design, for
+measuring what each part of the kernel costs); a default build contains none of them and ``fo_tune_set`` refuses
+their variant numbers.
 """
 from __future__ import annotations
 
@@ -75,6 +78,7 @@ def _run_hipcc(cmd: list, src: str, verbose: bool) -> None:
 def _compile_one(hipcc: str, src: str, extra: list, force: bool, verbose: bool) -> str:
     stem = os.path.splitext(src)[0]
     obj = os.path.join(OBJ_DIR, stem + ".o")
+    extra = extra + _EXTRA_DEFINES
     src_path = os.path.join(CSRC, src)
     stale = force or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(src_path), _newest_header_mtime())
     if not stale:
@@ -85,13 +89,18 @@ def _compile_one(hipcc: str, src: str, extra: list, force: bool, verbose: bool) 
     # Kernels with inline-assembly MFMAs: first without wait states in front of the MFMAs of the inner loops, keeping
     # the device assembly, which is then checked for the hazards the compiler cannot see inside an asm statement. If the
     # check finds one, compile again with the wait states.
-    from .asm_lint import lint_file
+    from .asm_lint import lint_file, lint_m0_file
     _run_hipcc([hipcc] + COMMON_FLAGS + extra + ["-DFO_MFMA_NOPS=0", "-save-temps=obj", "-c", src_path, "-o", obj], src, verbose)
     asm = os.path.join(OBJ_DIR, f"{stem}-hip-amdgcn-amd-amdhsa-{ARCH}.s")
     problems = lint_file(asm, ASM_LINTED[src]) if os.path.exists(asm) else [f"{asm} was not produced"]
+    # the direct-to-LDS copies are inline assembly too: M0 written and read back to back has no fallback build, it is
+    # an error in the source
+    m0_problems = lint_m0_file(asm) if os.path.exists(asm) else []
     for f in os.listdir(OBJ_DIR):           # the other intermediate files are large and of no further use
         if f.startswith(stem + "-") or f.startswith(stem + ".hip-"):
             os.remove(os.path.join(OBJ_DIR, f))
+    if m0_problems:
+        raise RuntimeError(f"{src}: {len(m0_problems)} LDS-DMA instruction(s) issued directly after a write of M0, e.g. {m0_problems[0]}")
     if problems:
         if verbose:
             print(f"{src}: {len(problems)} MFMA hazard(s) without wait states, e.g. {problems[0]}\n  -> compiling with wait states", flush=True)
@@ -101,10 +110,22 @@ def _compile_one(hipcc: str, src: str, extra: list, force: bool, verbose: bool) 
     return obj
 
 
-def build_library(force: bool = False, verbose: bool = True) -> str:
+_EXTRA_DEFINES: list = []
+
+
+def build_library(force: bool = False, verbose: bool = True, ablations: bool = False) -> str:
     """Compiles every HIP source for gfx950 and links the shared library. Returns the library path."""
+    global _EXTRA_DEFINES
+    _EXTRA_DEFINES = ["-DFO_ABLATIONS=1"] if ablations else []
     hipcc = _hipcc()
     os.makedirs(OBJ_DIR, exist_ok=True)
+    # objects compiled with other defines than this build's (an ablation build before a default one) are stale
+    stamp = os.path.join(OBJ_DIR, "defines.txt")
+    want = " ".join(_EXTRA_DEFINES)
+    if not os.path.exists(stamp) or open(stamp).read() != want:
+        force = True
+        with open(stamp, "w") as f:
+            f.write(want)
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
         objs = list(ex.map(lambda kv: _compile_one(hipcc, kv[0], kv[1], force, verbose), SOURCES.items()))
     need_link = force or not os.path.exists(LIB_PATH) or any(os.path.getmtime(o) > os.path.getmtime(LIB_PATH) for o in objs)
@@ -119,4 +140,4 @@ def build_library(force: bool = False, verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    print(build_library(force="--force" in sys.argv))
+    print(build_library(force="--force" in sys.argv or "--ablations" in sys.argv, ablations="--ablations" in sys.argv))

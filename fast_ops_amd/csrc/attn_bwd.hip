@@ -980,15 +980,16 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   AttnBwdParams q = p;
   {
     const int64_t bytes_head = 2 * ((int64_t)p.Sq + p.Sk) * D * 2;
-    int64_t group = g_attn_bwd_order >= 0 ? g_attn_bwd_order : bytes_head * n_bh <= (256ll << 20) ? n_bh : ((64ll << 20) / bytes_head) & ~7ll;
-    if (g_attn_bwd_order < 0 && group < 8) group = 8;
+    const int order = tune(g_attn_bwd_order);
+    int64_t group = order >= 0 ? order : bytes_head * n_bh <= (256ll << 20) ? n_bh : ((64ll << 20) / bytes_head) & ~7ll;
+    if (order < 0 && group < 8) group = 8;
     if (group <= 0 || group > n_bh) group = n_bh;
     q.head_group = (int)group;
   }
   // (delta is computed by the dQ kernel, which the dK/dV kernel follows)
   attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(q);
   // attn_bwd.variant 0 selects the plain dK/dV kernel everywhere (tests compare the two)
-  if (!DROP && !BIAS && g_attn_bwd_variant != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(q);
+  if (!DROP && !BIAS && tune(g_attn_bwd_variant) != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(q);
   else attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(q);
   return launch_status();
 }

@@ -32,16 +32,19 @@ __device__ __forceinline__ float half_swap(float x) {
 
 // 16 bytes per lane, global -> LDS without passing through registers. LDS receives the 64 lanes' pieces back to back
 // starting at `dst` (wave-uniform); the global address is per lane.
+// An LDS-DMA instruction reads M0 (the LDS destination) and needs one wait state after the scalar instruction that
+// wrote it. The compiler adds that s_nop for its own builtin; inside an asm statement nobody does, so it is spelled out
+// here, and the build's assembly check (asm_lint.py) verifies it for every kernel.
 // (hipcc also parses device functions in its host pass, where GCN assembly cannot be checked: the bodies exist in the
 // device pass only.)
 __device__ __forceinline__ void dma16_uniform_base(const void* base, uint32_t byte_off, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(byte_off), "s"(base) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(byte_off), "s"(base) : "memory", "m0");
 #endif
 }
 __device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
 #endif
 }
 
@@ -98,7 +101,7 @@ __device__ __forceinline__ void load_bias4(const E* at, float* out) {
 // the same with 4 bytes per lane (LDS receives 256 bytes)
 __device__ __forceinline__ void dma4_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
 #endif
 }
 

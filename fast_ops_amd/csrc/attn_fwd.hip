@@ -47,6 +47,7 @@ struct AttnParams {
   BiasParams bias;                      // used by the kernels instantiated with bias only
 };
 
+constexpr int64_t kMaxRowStride = 1ll << 24;   // elements; see attn_fwd_impl
 constexpr float kLazyLog2 = 8.0f;   // how far (in log2 units) a tile maximum may exceed the reference before a rescale
 
 template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false>
@@ -1070,47 +1071,55 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
   // 512 heads of 1 MiB in one group the kernel is bound by HBM (0.90 ms against 0.67 ms).
   AttnParams q = p;
   const int64_t kv_bytes_head = (int64_t)p.Sk * D * 2 * 2, n_bh_x = ((int64_t)p.B * p.H) >> 3;
-  int64_t group = g_attn_order >= 0 ? g_attn_order : 8 * n_bh_x * kv_bytes_head <= (256ll << 20) ? n_bh_x : (64ll << 20) / (8 * kv_bytes_head);
-  if (g_attn_order < 0 && group < 1) group = 1;
+  const int order = tune(g_attn_order);
+  int64_t group = order >= 0 ? order : 8 * n_bh_x * kv_bytes_head <= (256ll << 20) ? n_bh_x : (64ll << 20) / (8 * kv_bytes_head);
+  if (order < 0 && group < 1) group = 1;
   if (group > n_bh_x) group = n_bh_x;
   q.heavy_first = CAUSAL ? (int)group : 0;
   attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS><<<grid, kWaves * 64, lds, stream>>>(q);
   return launch_status();
 }
 
-// variant bit 0: 1 = exact (eager) rescale instead of the lazy one. Variants 2..7 are timing ablations that produce
-// WRONG results (bit 1: keep re-using the first tiles instead of copying new ones; bit 2: no exponentials).
+// Which kernel a call takes: FO_ATTN_KERNEL_ROWS128 / _ROWS128_EXACT (the 128-row kernel with the lazily raised or the
+// exact running maximum), FO_ATTN_KERNEL_ROWS256_W8 / _W4 (the 256-row kernel, eight waves x 32 rows or four x 64).
+// `forced` is the value of attn.variant (-1: the library's choice). Values from 256 on are timing ablations and exist
+// only in a build with FO_ABLATIONS.
+static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, int forced) {
+  // dropout and bias run on the 128-row kernel
+  if (p.bias.ptr != nullptr || dropout) return FO_ATTN_KERNEL_ROWS128;
+  // The 256-row kernel addresses a head's keys with 32-bit byte offsets ...
+  const bool wide_ok = (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
+  // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
+  // 128-row kernel, with four times as many workgroups, fills the chip better
+  static const int n_cu = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256; return n; }();
+  const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
+  // (causal, up to 2048 queries: a 256-row block is a large part of the triangle, and the 128-row kernel with its finer
+  // blocks, heaviest first, is 10-20 % faster at 1024 queries and equal or a few per cent faster at 2048)
+  int v = forced < 0 ? (wide_ok && wide_wgs >= n_cu && !(causal && p.Sq <= 2048) ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128) : forced;
+  if (v >= 256) return v;
+  if (!wide_ok && v >= 16) v = FO_ATTN_KERNEL_ROWS128;
+  if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128) v = FO_ATTN_KERNEL_ROWS128;   // the four-wave form exists for head_dim 128 only
+  return v;
+}
+
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
-  // dropout and bias run on the 128-row kernel
   if (p.bias.ptr != nullptr) {
     if (dropout) return causal ? launch_one<T, D, true, true, 0, true, true>(p, stream) : launch_one<T, D, false, true, 0, true, true>(p, stream);
     return causal ? launch_one<T, D, true, true, 0, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, true>(p, stream);
   }
   if (dropout) return causal ? launch_one<T, D, true, true, 0, true>(p, stream) : launch_one<T, D, false, true, 0, true>(p, stream);
-  // default: the wide kernel (eight waves x 32 rows)
-  // (it addresses a head's keys with 32-bit byte offsets)
-  // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
-  // 128-row kernel, with four times as many workgroups, fills the chip better
-  static const int n_cu = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256; return n; }();
-  const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
-  const bool wide_ok = (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
-  // (causal, up to 2048 queries: a 256-row block is a large part of the triangle, and the 128-row kernel with its finer
-  // blocks, heaviest first, is 10-20 % faster at 1024 queries and equal or a few per cent faster at 2048)
-  int v = g_attn_variant < 0 ? (wide_ok && wide_wgs >= n_cu && !(causal && p.Sq <= 2048) ? 16 : 0) : g_attn_variant;
-  if (!wide_ok && v >= 16) v = 0;
-  if constexpr (D == 64) {
-    if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
-    if (v >= 16) v = 0;
-  }
+  const int v = choose_kernel(p, D, causal, dropout, tune(g_attn_variant));
+  if (v == FO_ATTN_KERNEL_ROWS256_W8) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
   if constexpr (D == 128) {
-    // 16: wide kernel, eight waves x 32 rows; 32: wide kernel, four waves x 64 rows
-    if (v == 16) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
-    if (v == 32) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
-    // timing ablations (WRONG results), non-causal only: 256 + bits for eight waves, 512 + bits for four.
-    // bit 0 no global->LDS copies, 1 no exponentials, 2 no LDS fragment reads,
-    // 5 no wait for copies, 6 no barrier
-    if constexpr (std::is_same<T, __bf16>::value) if (v >= 256 && !causal) {
+    if (v == FO_ATTN_KERNEL_ROWS256_W4) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
+  }
+#if defined(FO_ABLATIONS)
+  // Timing ablations (WRONG results by design; bf16, head_dim 128 only). 256-row kernel, non-causal: 256 + bits for eight
+  // waves, 512 + bits for four; bit 0 no global->LDS copies, 1 no exponentials, 2 no LDS fragment reads, 5 no wait for
+  // copies, 6 no barrier. 128-row kernel, causal: 2..11.
+  if constexpr (D == 128 && std::is_same<T, __bf16>::value) {
+    if (v >= 256 && !causal) {
       switch (v) {
         case 256 + 1: return launch_wide<T, D, false, 1, 1>(p, stream);
         case 256 + 2: return launch_wide<T, D, false, 1, 2>(p, stream);
@@ -1124,18 +1133,20 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
         default: return FO_ERR_UNSUPPORTED;
       }
     }
-  }
-  if (D == 128 && causal && sizeof(T) == 2) {
-    switch (v >> 1) {
-      case 1: return launch_one<T, D, true, true, 1>(p, stream);
-      case 2: return launch_one<T, D, true, true, 2>(p, stream);
-      case 3: return launch_one<T, D, true, true, 3>(p, stream);
-      case 4: return launch_one<T, D, true, true, 5>(p, stream);
-      case 5: return launch_one<T, D, true, true, 7>(p, stream);
-      default: break;
+    if (causal) {
+      switch (v >> 1) {
+        case 1: return launch_one<T, D, true, true, 1>(p, stream);
+        case 2: return launch_one<T, D, true, true, 2>(p, stream);
+        case 3: return launch_one<T, D, true, true, 3>(p, stream);
+        case 4: return launch_one<T, D, true, true, 5>(p, stream);
+        case 5: return launch_one<T, D, true, true, 7>(p, stream);
+        default: break;
+      }
     }
   }
-  const bool lazy = (v & 1) == 0;
+#endif
+  if (v != FO_ATTN_KERNEL_ROWS128 && v != FO_ATTN_KERNEL_ROWS128_EXACT) return FO_ERR_UNSUPPORTED;
+  const bool lazy = v == FO_ATTN_KERNEL_ROWS128;
   if (causal) return lazy ? launch_one<T, D, true, true, 0>(p, stream) : launch_one<T, D, true, false, 0>(p, stream);
   return lazy ? launch_one<T, D, false, true, 0>(p, stream) : launch_one<T, D, false, false, 0>(p, stream);
 }
@@ -1165,6 +1176,9 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   }
   if (os[0] == 0 && B > 1) return FO_ERR_BAD_STRIDE;
   if (os[1] == 0 && H > 1) return FO_ERR_BAD_STRIDE;
+  // the 128-row kernel addresses the 64 rows of a key tile with 32-bit byte offsets (the 256-row kernel, whose offsets
+  // span a whole head, is chosen only where they fit): 63 * stride * 2 bytes must stay below 2^32
+  if (ks[2] >= kMaxRowStride || vs[2] >= kMaxRowStride) return FO_ERR_BAD_STRIDE;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15u) return FO_ERR_MISALIGNED;
   if (lse && ((uintptr_t)lse & 3u)) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;   // also rejects NaN
@@ -1198,6 +1212,19 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == FO_DTYPE_BF16) return D == 128 ? launch<__bf16, 128>(p, causal != 0, drop, s) : launch<__bf16, 64>(p, causal != 0, drop, s);
   return D == 128 ? launch<_Float16, 128>(p, causal != 0, drop, s) : launch<_Float16, 64>(p, causal != 0, drop, s);
+}
+
+extern "C" int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* ks, const int64_t* vs,
+                                  int causal, int has_bias, int has_dropout) {
+  if (!ks || !vs) return FO_ERR_NULL_POINTER;
+  if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
+  if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return FO_ERR_BAD_SHAPE;
+  if (ks[2] < D || vs[2] < D || ks[2] >= kMaxRowStride || vs[2] >= kMaxRowStride) return FO_ERR_BAD_STRIDE;
+  AttnParams p = {};
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  for (int i = 0; i < 3; ++i) { p.ks[i] = ks[i]; p.vs[i] = vs[i]; }
+  p.bias.ptr = has_bias ? (const void*)ks : nullptr;   // (only tested against NULL)
+  return choose_kernel(p, D, causal != 0, has_dropout != 0, tune(g_attn_variant));
 }
 
 extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,

@@ -4,11 +4,11 @@
 #include "common.hpp"
 
 namespace fo {
-int g_lion_variant = -1;
-int g_attn_variant = -1;
-int g_attn_bwd_variant = -1;
-int g_attn_order = -1;
-int g_attn_bwd_order = -1;
+std::atomic<int> g_lion_variant{-1};
+std::atomic<int> g_attn_variant{-1};
+std::atomic<int> g_attn_bwd_variant{-1};
+std::atomic<int> g_attn_order{-1};
+std::atomic<int> g_attn_bwd_order{-1};
 }  // namespace fo
 
 extern "C" const char* fo_strerror(int status) {
@@ -31,9 +31,25 @@ extern "C" int fo_version(void) { return 1000; }
 extern "C" int fo_tune_set(const char* key, int value) {
   if (!key) return FO_ERR_NULL_POINTER;
   if (value < -1) return FO_ERR_UNSUPPORTED;
-  if (strcmp(key, "lion.variant") == 0) { fo::g_lion_variant = value; return FO_OK; }
-  if (strcmp(key, "attn.variant") == 0) { fo::g_attn_variant = value; return FO_OK; }
-  if (strcmp(key, "attn_bwd.variant") == 0) { fo::g_attn_bwd_variant = value; return FO_OK; }
+  // Every accepted value selects a kernel (or a workgroup order) that computes the same function; values that stand
+  // for timing ablations with wrong results exist only in a library built with FO_ABLATIONS.
+  if (strcmp(key, "lion.variant") == 0) {
+    if (value >= 32) return FO_ERR_UNSUPPORTED;                       // launch shapes 0..31
+    fo::g_lion_variant = value; return FO_OK;
+  }
+  if (strcmp(key, "attn.variant") == 0) {
+    // FO_ATTN_KERNEL_*: 0 / 1 = 128-row kernel with the lazy / the exact rescale, 16 / 32 = 256-row kernel, 8 / 4 waves
+    bool ok = value == -1 || value == 0 || value == 1 || value == 16 || value == 32;
+#if defined(FO_ABLATIONS)
+    ok = true;
+#endif
+    if (!ok) return FO_ERR_UNSUPPORTED;
+    fo::g_attn_variant = value; return FO_OK;
+  }
+  if (strcmp(key, "attn_bwd.variant") == 0) {
+    if (value > 1) return FO_ERR_UNSUPPORTED;                         // 0 = plain dK/dV kernel, 1 = pipelined (default)
+    fo::g_attn_bwd_variant = value; return FO_OK;
+  }
   if (strcmp(key, "attn.order") == 0) { fo::g_attn_order = value; return FO_OK; }
   if (strcmp(key, "attn_bwd.order") == 0) { fo::g_attn_bwd_order = value; return FO_OK; }
   return FO_ERR_UNSUPPORTED;
@@ -41,10 +57,17 @@ extern "C" int fo_tune_set(const char* key, int value) {
 
 extern "C" int fo_tune_get(const char* key) {
   if (!key) return FO_ERR_NULL_POINTER;
-  if (strcmp(key, "lion.variant") == 0) return fo::g_lion_variant;
-  if (strcmp(key, "attn.variant") == 0) return fo::g_attn_variant;
-  if (strcmp(key, "attn_bwd.variant") == 0) return fo::g_attn_bwd_variant;
-  if (strcmp(key, "attn.order") == 0) return fo::g_attn_order;
-  if (strcmp(key, "attn_bwd.order") == 0) return fo::g_attn_bwd_order;
+  if (strcmp(key, "lion.variant") == 0) return fo::tune(fo::g_lion_variant);
+  if (strcmp(key, "attn.variant") == 0) return fo::tune(fo::g_attn_variant);
+  if (strcmp(key, "attn_bwd.variant") == 0) return fo::tune(fo::g_attn_bwd_variant);
+  if (strcmp(key, "attn.order") == 0) return fo::tune(fo::g_attn_order);
+  if (strcmp(key, "attn_bwd.order") == 0) return fo::tune(fo::g_attn_bwd_order);
+  if (strcmp(key, "build.ablations") == 0) {
+#if defined(FO_ABLATIONS)
+    return 1;
+#else
+    return 0;
+#endif
+  }
   return FO_ERR_UNSUPPORTED;
 }

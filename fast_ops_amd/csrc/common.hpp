@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/fastops.h"
 
 namespace fo {
@@ -18,12 +20,14 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 
-// variant selectors set through fo_tune_set (-1 = default)
-extern int g_lion_variant;
-extern int g_attn_variant;
-extern int g_attn_bwd_variant;
-extern int g_attn_bwd_order;   // attention backward: -1 automatic, 0 all heads in one group, n > 0 groups of n heads
-extern int g_attn_order;   // 128-row attention kernel, causal: -1 automatic, 0 head by head, n > 0 heaviest query blocks first within groups of n heads per XCD
+// variant selectors set through fo_tune_set (-1 = default). Atomic so that a host thread that sets one while another
+// thread launches reads a whole value; an entry point reads each selector once per call.
+extern std::atomic<int> g_lion_variant;
+extern std::atomic<int> g_attn_variant;
+extern std::atomic<int> g_attn_bwd_variant;
+extern std::atomic<int> g_attn_bwd_order;   // attention backward: -1 automatic, 0 all heads in one group, n > 0 groups of n heads
+extern std::atomic<int> g_attn_order;   // 128-row attention kernel, causal: -1 automatic, 0 head by head, n > 0 heaviest query blocks first within groups of n heads per XCD
+inline int tune(const std::atomic<int>& v) { return v.load(std::memory_order_relaxed); }
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? FO_OK : FO_ERR_LAUNCH; }
 

@@ -267,7 +267,8 @@ extern "C" int fo_lion_step(const fo_lion_chunk* chunks_dev, int64_t n_chunks, c
   if (n_chunks == 0) return FO_OK;
   if (!chunks_dev) return FO_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(chunks_dev) & 7u) return FO_ERR_MISALIGNED;
-  const int v = (g_lion_variant < 0 || g_lion_variant >= kLionVariants) ? kLionDefaultVariant : g_lion_variant;
+  const int tv = tune(g_lion_variant);
+  const int v = (tv < 0 || tv >= kLionVariants) ? kLionDefaultVariant : tv;
   return launch_variant(v, chunks_dev, n_chunks, nullptr, nullptr, nullptr, 0, to_c(consts), static_cast<hipStream_t>(stream));
 }
 
@@ -278,6 +279,7 @@ extern "C" int fo_lion_update(float* p, const float* g, uint16_t* m, int64_t num
   if (!p || !g || !m) return FO_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(p) & 3u) || (reinterpret_cast<uintptr_t>(g) & 3u) || (reinterpret_cast<uintptr_t>(m) & 1u))
     return FO_ERR_MISALIGNED;
-  const int v = (g_lion_variant < 0 || g_lion_variant >= kLionVariants) ? kLionDefaultVariant : g_lion_variant;
+  const int tv = tune(g_lion_variant);
+  const int v = (tv < 0 || tv >= kLionVariants) ? kLionDefaultVariant : tv;
   return launch_variant(v, nullptr, 0, p, g, m, numel, to_c(consts), static_cast<hipStream_t>(stream));
 }

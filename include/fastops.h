@@ -44,9 +44,13 @@ const char* fo_strerror(int status);
 /* Library ABI version: major*1000 + minor. */
 int fo_version(void);
 
-/* Tuning hook for benchmarks and profiling: selects a kernel variant by name ("lion.variant", "attn.variant").
- * The defaults are the measured best; value -1 restores the default. Returns FO_OK or FO_ERR_UNSUPPORTED for an
- * unknown key or value. Process-global and not synchronised with calls in flight. No reference counterpart. */
+/* Tuning hook for benchmarks, profiling and tests: selects a kernel variant or a workgroup order by name
+ * ("lion.variant", "attn.variant", "attn_bwd.variant", "attn.order", "attn_bwd.order"). Every value it accepts selects
+ * code that computes the same function as the default; value -1 restores the default (the measured best). Returns
+ * FO_OK, or FO_ERR_UNSUPPORTED for an unknown key or a value that selects nothing. The settings are process-global
+ * atomics: a call reads each one once, a call already issued is not affected. fo_tune_get additionally answers
+ * "build.ablations" (1 if the library was built with the timing ablations of the attention forward, which produce
+ * wrong results by design and which a default build does not contain; 0 otherwise). No reference counterpart. */
 int fo_tune_set(const char* key, int value);
 int fo_tune_get(const char* key);
 
@@ -68,13 +72,28 @@ int fo_tune_get(const char* key);
  *   dtype        FO_DTYPE_F16 or FO_DTYPE_BF16, for q, k, v and o alike
  *
  * Requirements checked here: D in {64, 128}; Sq, Sk >= 1; softmax_scale finite and > 0; base pointers and row strides
- * multiples of 16 bytes.
+ * multiples of 16 bytes; sequence strides of k and v below 2^24 elements (FO_ERR_BAD_STRIDE otherwise: the kernels
+ * address the rows of a key tile with 32-bit byte offsets).
  */
 int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                 int B, int H, int Sq, int Sk, int D,
                 const int64_t* q_strides_host, const int64_t* k_strides_host,
                 const int64_t* v_strides_host, const int64_t* o_strides_host,
                 float softmax_scale, int causal, int dtype, void* stream);
+
+/* Which kernel fo_attn_fwd (or _dropout / _ex, with has_dropout / has_bias non-zero) launches for a call of this shape
+ * on the current device with the current "attn.variant": one of the FO_ATTN_KERNEL_* codes below, or a negative
+ * fo_status where fo_attn_fwd would reject the shape. Launches nothing. The choice depends on the number of compute
+ * units of the device that was current when the library first chose (read once per process). No reference counterpart:
+ * the reference has one kernel (flash_attention_fwd.cu:164-177); tests use this to assert which code they covered. */
+enum {
+  FO_ATTN_KERNEL_ROWS128 = 0,         /* 128 query rows per workgroup, reference maximum raised lazily */
+  FO_ATTN_KERNEL_ROWS128_EXACT = 1,   /* the same with the exact running maximum of flash_attention_triton.py:200-213 */
+  FO_ATTN_KERNEL_ROWS256_W8 = 16,     /* 256 query rows per workgroup, eight waves x 32 rows */
+  FO_ATTN_KERNEL_ROWS256_W4 = 32      /* 256 query rows per workgroup, four waves x 64 rows (head_dim 128 only) */
+};
+int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* k_strides_host, const int64_t* v_strides_host,
+                       int causal, int has_bias, int has_dropout);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * FlashAttention backward: dQ, dK, dV.

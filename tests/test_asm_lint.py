@@ -36,3 +36,19 @@ def test_reading_an_mfma_result_too_early_is_flagged():
     to_v = "v_mfma_f32_32x32x16_f16 v[16:31], v[0:3], v[4:7], 0"
     assert _lint(f"{to_v}\nv_mul_f32_e32 v40, v41, v17")
     assert not _lint(f"{to_v}\ns_nop 7\ns_nop 7\nv_mul_f32_e32 v40, v41, v17")
+
+
+def test_lds_dma_right_after_an_m0_write_is_flagged():
+    from fast_ops_amd.asm_lint import lint_m0_function
+
+    lint = lambda text: lint_m0_function(text.strip().splitlines(), "k")
+    dma = "global_load_lds_dwordx4 v2, s[6:7]"
+    assert lint(f"s_mov_b32 m0, s5\n{dma}")                              # no wait state
+    assert lint(f"s_add_u32 m0, s5, 0x400\n{dma}")                       # any scalar write of M0 counts
+    assert lint(f"s_mov_b32 m0, s5\n.LBB0_3:\n{dma}")                    # a label in between changes nothing
+    assert lint("s_mov_b32 m0, s5\nbuffer_load_dword v1, s[8:11], 0 offen lds")
+    assert not lint(f"s_mov_b32 m0, s5\ns_nop 0\n{dma}")                 # one wait state: enough
+    assert not lint(f"s_mov_b32 m0, s5\nv_add_u32_e32 v2, v2, v3\n{dma}")
+    assert not lint(f"s_mov_b32 s4, s5\n{dma}")                          # not M0
+    assert not lint("s_mov_b32 m0, s5\nbuffer_load_dword v1, s[8:11], 0 offen")   # not an LDS-DMA
+    assert not lint("s_mov_b32 m0, s5\nds_read_b128 v[0:3], v30")

@@ -151,10 +151,54 @@ def test_tune_hook():
     assert lib.fo_tune_set(b"lion.variant", -1) == 0
     assert lib.fo_tune_set(b"no.such.key", 1) == -8
     # every key the kernels read: default -1 (the library's choice), settable, readable
-    for key in (b"attn.variant", b"attn_bwd.variant", b"attn.order", b"attn_bwd.order"):
+    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn_bwd.order", 2)):
         assert lib.fo_tune_get(key) == -1
-        assert lib.fo_tune_set(key, 2) == 0 and lib.fo_tune_get(key) == 2
+        assert lib.fo_tune_set(key, value) == 0 and lib.fo_tune_get(key) == value
         assert lib.fo_tune_set(key, -1) == 0 and lib.fo_tune_get(key) == -1
+
+
+def test_tune_hook_accepts_only_kernels_that_compute_the_function():
+    # the shipped library holds no timing ablations (kernel variants that leave work out): their numbers select nothing
+    lib = _lib.load()
+    assert lib.fo_tune_get(b"build.ablations") == 0
+    for ok in (-1, 0, 1, 16, 32):
+        assert lib.fo_tune_set(b"attn.variant", ok) == 0
+    for bad in (2, 3, 7, 8, 15, 17, 33, 257, 258, 260, 263, 320, 384, 519, 520, 640, -2):
+        assert lib.fo_tune_set(b"attn.variant", bad) == -8, bad
+        assert lib.fo_tune_get(b"attn.variant") == 32          # a refused value changes nothing
+    assert lib.fo_tune_set(b"attn.variant", -1) == 0
+    assert lib.fo_tune_set(b"attn_bwd.variant", 2) == -8
+    assert lib.fo_tune_set(b"lion.variant", 32) == -8
+
+
+def test_attn_kernel_query_and_stride_limit_without_device_work():
+    lib = _lib.load()
+    I3 = ctypes.c_int64 * 3
+    dense = lambda S, D: I3(S * D * 4, S * D, D)
+    k = lambda B, H, Sq, Sk, D, causal, bias=0, drop=0, ks=None: lib.fo_attn_fwd_kernel(
+        B, H, Sq, Sk, D, ks or dense(Sk, D), ks or dense(Sk, D), causal, bias, drop)
+    # small shapes, bias and dropout always take the 128-row kernel, whatever the device
+    assert k(1, 1, 128, 128, 64, 0) == _lib.FO_ATTN_KERNEL_ROWS128
+    assert k(2, 16, 8192, 8192, 128, 1, bias=1) == _lib.FO_ATTN_KERNEL_ROWS128
+    assert k(2, 16, 8192, 8192, 128, 1, drop=1) == _lib.FO_ATTN_KERNEL_ROWS128
+    # forced choices are honoured where the kernel exists
+    assert lib.fo_tune_set(b"attn.variant", 32) == 0
+    try:
+        assert k(1, 1, 512, 512, 128, 0) == _lib.FO_ATTN_KERNEL_ROWS256_W4
+        assert k(1, 1, 512, 512, 64, 0) == _lib.FO_ATTN_KERNEL_ROWS128          # no four-wave form for head_dim 64
+        assert lib.fo_tune_set(b"attn.variant", 1) == 0
+        assert k(1, 1, 512, 512, 64, 1) == _lib.FO_ATTN_KERNEL_ROWS128_EXACT
+    finally:
+        lib.fo_tune_set(b"attn.variant", -1)
+    assert k(1, 1, 128, 128, 72, 0) == -3 and k(0, 1, 128, 128, 64, 0) == -4
+    assert lib.fo_attn_fwd_kernel(1, 1, 128, 128, 64, None, dense(128, 64), 0, 0, 0) == -1
+    # K/V row strides of 2^24 elements and more do not fit the kernels' 32-bit tile offsets: rejected, not wrapped
+    wide_rows = I3(0, 0, 1 << 24)
+    assert k(1, 1, 128, 128, 64, 0, ks=wide_rows) == -5
+    ok_ptr = 0x1000
+    s = dense(128, 64)
+    assert lib.fo_attn_fwd(ok_ptr, ok_ptr, ok_ptr, ok_ptr, None, 1, 1, 128, 128, 64, s, wide_rows, s, s, 0.125, 0, 1, None) == -5
+    assert lib.fo_attn_fwd(ok_ptr, ok_ptr, ok_ptr, ok_ptr, None, 1, 1, 128, 128, 64, s, s, wide_rows, s, 0.125, 0, 1, None) == -5
 
 
 def test_python_surfaces_validate_like_the_reference():
