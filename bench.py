@@ -1,12 +1,23 @@
 """Benchmark of the two hot paths on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--path both|attn|lion] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle N] [--path both|attn|lion|copy] [--no-cpu-baseline]
+                    [--headline-only]
 
 Prints ONE JSON line. The headline value is the attention forward throughput at B=2 H=16 S=8192 D=128 bf16 causal
 (FLOPs counted as 2*B*H*S^2*D); the fused Lion step over 1,308,622,848 fp32 parameters with bf16 momentum (16 bytes
 per parameter) is reported in the "lion" object of the same line, each with its roofline and a CPU baseline timed on
-this host's cores. The attention backward of the same shape is reported in "attn_bwd", and the rate of the vendor
-library's plain bf16 GEMM on random operands on the same box in "library_gemm" (what MFMA code reaches here at all).
+this host's cores. Beside them, not part of the headline: the attention backward of the same shape ("attn_bwd"), the
+other three benchmark configurations ("configs": GPT-2-small attention forward, GPT-2-small Lion, fp16 non-causal
+attention forward at B=16 H=32 S=2048 D=128), and the rate of the vendor library's plain bf16 GEMM on random operands
+on the same box ("library_gemm": what MFMA code reaches here at all).
+
+Every timed section is preceded by a clock-settle phase of --settle launches of the same step (default 100, reported
+under "settle"), which is not part of the W warm-up steps: after idling, the GPU's clocks take a few dozen launches
+to settle (the per-launch time of the attention kernel wanders by 25 % over the first 30 launches, then stays within
+1 %), so without it the result would depend on the caller's --warmup.
+
+All inputs are drawn from a CPU torch.Generator in fp32 with the seeds the configurations name, cast, and copied to the
+GPU before timing starts; nothing crosses PCIe in a timed region.
 """
 import argparse
 import json
@@ -20,6 +31,8 @@ if ROOT not in sys.path:
 
 PEAK_MFMA_TFLOPS = 2500.0     # MI355X dense bf16/fp16
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload, recorded in "
+                  "profiles/hbm_traffic_pmc_attn_S8192_lion_1p3B.txt; a constant read from profiles/hbm_traffic.json, not measured by this run")
 
 
 def _measured_traffic(key):
@@ -32,41 +45,99 @@ def _measured_traffic(key):
         return None
 
 
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def _events(n):
     import torch
 
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def _time_steps(step, steps, warmup):
-    """W untimed steps, then K timed steps bracketed by synchronize; per-launch durations from HIP events recorded on
-    the stream the kernels are launched on (torch's current stream)."""
+def _settle(step, launches):
+    """`launches` untimed-for-the-result launches of `step` so that the clocks are where a sustained run has them; the
+    first and last per-launch times are reported to show what the phase did."""
     import torch
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    ev = _events(steps + 1)
-    t0 = time.perf_counter()
+    if launches <= 0:
+        return {"launches": 0}
+    ev = _events(launches + 1)
     ev[0].record()
-    for i in range(steps):
+    for i in range(launches):
         step()
         ev[i + 1].record()
     torch.cuda.synchronize()
+    ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(launches)]
+    k = max(1, min(5, launches // 2))
+    return {"launches": launches, "ms_first": sum(ms[:k]) / k, "ms_last": sum(ms[-k:]) / k, "ms_max": max(ms)}
+
+
+def _time_steps(step, steps, warmup, settle=0, before_each=None):
+    """`settle` clock-settle launches, W untimed steps, then K timed steps bracketed by synchronize; per-launch durations
+    from HIP events recorded on the stream the kernels are launched on (torch's current stream). `before_each(i)`, if
+    given, runs before timed step i outside its pair of events (fresh inputs for the step)."""
+    import torch
+
+    info = _settle(step, settle)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    starts, ends = _events(steps), _events(steps)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        if before_each is not None:
+            before_each(i)
+        starts[i].record()
+        step()
+        ends[i].record()
+    torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    per_launch = [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
-    return wall_ms / steps, sum(per_launch) / steps, min(per_launch)
+    per_launch = [starts[i].elapsed_time(ends[i]) for i in range(steps)]
+    return wall_ms / steps, sum(per_launch) / steps, min(per_launch), info
 
 
-def bench_attention(steps, warmup, cpu_baseline):
+def _attn_inputs(B, H, S, D, dtype, dev, seed=0):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    return tuple(torch.randn(B, H, S, D, generator=g).to(dtype).to(dev) for _ in range(3)), g
+
+
+def _attn_rate(B, H, S, D, dtype, causal, steps, warmup, settle):
+    """One attention-forward configuration through multi_head_attention: (wall ms per step, kernel ms, min, settle info,
+    FLOPs, which kernel ran)."""
+    import ctypes
+
+    import torch
+
+    from fast_ops.flash_attention.flash_attention import multi_head_attention
+    from fast_ops_amd import _lib
+
+    (q, k, v), _ = _attn_inputs(B, H, S, D, dtype, "cuda:0")
+    scale = 1.0 / (D ** 0.5)
+    flops = (2.0 if causal else 4.0) * B * H * S * S * D
+    ms_step, ms_kernel, ms_min, info = _time_steps(lambda: multi_head_attention(q, k, v, causal=causal, softmax_scale=scale, return_lse=True), steps, warmup, settle)
+    I3 = ctypes.c_int64 * 3
+    kernel = _lib.load().fo_attn_fwd_kernel(B, H, S, S, D, I3(*k.stride()[:3]), I3(*v.stride()[:3]), int(causal), 0, 0)
+    return ms_step, ms_kernel, ms_min, info, flops, {0: "rows128", 1: "rows128_exact", 16: "rows256_w8", 32: "rows256_w4"}.get(kernel, str(kernel))
+
+
+def bench_attention(steps, warmup, settle, cpu_baseline, extras):
     import torch
 
     from fast_ops.flash_attention.flash_attention import multi_head_attention
 
     B, H, S, D = 2, 16, 8192, 128
     dev = "cuda:0"
-    g = torch.Generator().manual_seed(0)
-    q, k, v = (torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev) for _ in range(3))
+    (q, k, v), g = _attn_inputs(B, H, S, D, torch.bfloat16, dev)
     scale = 1.0 / (D ** 0.5)
     flops = 2.0 * B * H * S * S * D      # causal-halved 4*B*H*S^2*D
     out = {}
@@ -74,42 +145,45 @@ def bench_attention(steps, warmup, cpu_baseline):
     def step():
         out["o"], out["lse"] = multi_head_attention(q, k, v, causal=True, softmax_scale=scale, return_lse=True)
 
-    ms_step, ms_kernel, ms_min = _time_steps(step, steps, warmup)
+    ms_step, ms_kernel, ms_min, info = _time_steps(step, steps, warmup, settle)
     res = {
         "value": flops / (ms_step * 1e-3) / 1e12,
         "ms_per_step": ms_step,
+        "settle": info,
         "roofline": {
             "bound": "mfma", "achieved": flops / (ms_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-            "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": _measured_traffic("attn"),
+            "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": _measured_traffic("attn"), "traffic_source": TRAFFIC_SOURCE,
             "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "flops_per_launch": flops,
         },
         "workload": f"attention fwd B={B} H={H} S={S} D={D} bf16 causal, scale 1/sqrt({D})",
     }
-    # the backward of the same workload (dQ, dK, dV; two launches), reported beside the headline, not part of it
-    from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided
+    if extras:
+        # the backward of the same workload (dQ, dK, dV; two launches), reported beside the headline, not part of it
+        from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided
 
-    go = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev)
-    o_fix, lse_fix = out["o"], out["lse"]
-    bwd_flops = 5.0 * B * H * S * S * D      # causal-halved 10*B*H*S^2*D (five GEMMs; the kernels recompute two more)
-    b_step, b_kernel, b_min = _time_steps(lambda: attn_bwd_strided(q, k, v, o_fix, lse_fix, go, (0, 1, 2, 3), True, scale), steps, warmup)
-    res["bwd"] = {
-        "value": bwd_flops / (b_step * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": b_step,
-        "roofline": {"bound": "mfma", "achieved": bwd_flops / (b_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": bwd_flops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": None,
-                     "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "flops_per_launch": bwd_flops},
-        "workload": "attention bwd (dQ + dK/dV kernels) of the same shape, FLOPs by the five-GEMM count",
-    }
-    # yardstick, not part of the headline: the vendor library's plain bf16 GEMM on the same box with the same kind of
-    # data. Under a full-chip MFMA load the clock follows the power drawn, which depends on the operand bits (all-zero
-    # operands run a third faster than random ones), so the published peak is not what random data can reach.
-    n = 8192
-    ga, gb = (torch.randn(n, n, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
-    _, g_kernel, _ = _time_steps(lambda: torch.matmul(ga, gb), 20, 20)
-    res["library_gemm"] = {
-        "value": 2.0 * n ** 3 / (g_kernel * 1e-3) / 1e12, "unit": "TFLOP/s", "frac_of_peak": 2.0 * n ** 3 / (g_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
-        "what": f"torch.matmul (hipBLASLt) bf16 {n}x{n}x{n}, standard normal operands, same box, timed after the attention runs",
-    }
-    del ga, gb
+        go = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev)
+        o_fix, lse_fix = out["o"], out["lse"]
+        bwd_flops = 5.0 * B * H * S * S * D      # causal-halved 10*B*H*S^2*D (five GEMMs; the kernels recompute two more)
+        b_step, b_kernel, b_min, b_info = _time_steps(lambda: attn_bwd_strided(q, k, v, o_fix, lse_fix, go, (0, 1, 2, 3), True, scale), steps, warmup, settle // 2)
+        res["bwd"] = {
+            "value": bwd_flops / (b_step * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": b_step, "settle": b_info,
+            "roofline": {"bound": "mfma", "achieved": bwd_flops / (b_kernel * 1e-3) / 1e12, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                         "frac": bwd_flops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "traffic": None,
+                         "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "flops_per_launch": bwd_flops},
+            "workload": "attention bwd (dQ + dK/dV kernels) of the same shape, FLOPs by the five-GEMM count",
+        }
+        del go, o_fix, lse_fix
+        # yardstick, not part of the headline: the vendor library's plain bf16 GEMM on the same box with the same kind of
+        # data. Under a full-chip MFMA load the clock follows the power drawn, which depends on the operand bits (all-zero
+        # operands run a third faster than random ones), so the published peak is not what random data can reach.
+        n = 8192
+        ga, gb = (torch.randn(n, n, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
+        _, g_kernel, _, _ = _time_steps(lambda: torch.matmul(ga, gb), 20, 20, settle // 2)
+        res["library_gemm"] = {
+            "value": 2.0 * n ** 3 / (g_kernel * 1e-3) / 1e12, "unit": "TFLOP/s", "frac_of_peak": 2.0 * n ** 3 / (g_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
+            "what": f"torch.matmul (hipBLASLt) bf16 {n}x{n}x{n}, standard normal operands, same box, timed after the attention runs",
+        }
+        del ga, gb
     if cpu_baseline:
         # bounded sample: all (batch, head) slices of the same workload through the oracle's fp32 vanilla path on all host
         # cores, stopped after about 15 s; the rate is that of the slices that were finished
@@ -127,38 +201,102 @@ def bench_attention(steps, warmup, cpu_baseline):
                 n_sl += 1
         dt = time.perf_counter() - t0
         res["cpu_baseline"] = {
-            "value": n_sl * 2.0 * S * S * D / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "value": n_sl * 2.0 * S * S * D / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "cpu_model": _cpu_model(), "kind": "port",
             "sample": f"{n_sl} of {B * H} (batch, head) slices of the same shape, fp32 vanilla softmax(QK^T)V on the host, {dt:.2f} s",
         }
+    del q, k, v
+    out.clear()
+    torch.cuda.empty_cache()
+    if extras:
+        # the other attention configurations: report only
+        res["configs"] = {}
+        for name, (b_, h_, s_, d_, dt_, causal_) in {
+            "2_attn_fwd_gpt2_small": (8, 12, 1024, 64, torch.bfloat16, True),
+            "5a_attn_fwd_throughput": (16, 32, 2048, 128, torch.float16, False),
+        }.items():
+            c_step, c_kernel, c_min, c_info, c_flops, c_k = _attn_rate(b_, h_, s_, d_, dt_, causal_, steps, warmup, settle)
+            res["configs"][name] = {
+                "workload": f"attention fwd B={b_} H={h_} S={s_} D={d_} {'bf16' if dt_ == torch.bfloat16 else 'fp16'} {'causal' if causal_ else 'non-causal'}",
+                "ms_per_step": c_step, "kernel_ms_avg": c_kernel, "kernel_ms_min": c_min, "value": c_flops / (c_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+                "frac": c_flops / (c_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": c_flops, "kernel": c_k, "settle": c_info,
+            }
+            torch.cuda.empty_cache()
     return res
 
 
-def bench_lion(steps, warmup, cpu_baseline):
+GPT2_SMALL_SHAPES = ([(50257, 768), (1024, 768)]
+                     + [s for _ in range(12) for s in [(768,), (768,), (768, 2304), (2304,), (768, 768), (768,), (768,), (768,), (768, 3072), (3072,), (3072, 768), (768,)]]
+                     + [(768,), (768,)])
+LION_LARGE_SHAPES = [(2048, 8192)] * 39 + [(8192, 2048)] * 39
+LION_HP = dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
+
+
+def _lion_setup(shapes, dev):
+    """Parameters ~ N(0, 0.02) and bf16 momentum ~ N(0, 1e-3) from a CPU generator seeded 0 (parameters first, then
+    momenta), gradients ~ N(0, 1e-2) from seed 1000 (the first step's); copied to the GPU."""
     import torch
 
     from fast_ops.lion.lion_optimizer import Lion
 
-    dev = "cuda:0"
-    shapes = [(2048, 8192)] * 39 + [(8192, 2048)] * 39
-    n_params = sum(a * b for a, b in shapes)
-    gen = torch.Generator(device=dev).manual_seed(0)
-    params = [torch.nn.Parameter(torch.randn(s, device=dev, generator=gen) * 0.02) for s in shapes]
-    hp = dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
-    opt = Lion(params, **hp)
+    gen = torch.Generator().manual_seed(0)
+    params = [torch.nn.Parameter((torch.randn(s, generator=gen) * 0.02).to(dev)) for s in shapes]
+    opt = Lion(params, **LION_HP)
     for p in params:
-        opt.state[p]["exp_avg"] = (torch.randn(p.shape, device=dev, generator=gen) * 1e-3).to(torch.bfloat16)
-        p.grad = torch.randn(p.shape, device=dev, generator=gen) * 1e-2
+        opt.state[p]["exp_avg"] = (torch.randn(p.shape, generator=gen) * 1e-3).to(torch.bfloat16).to(dev)
+    ggen = torch.Generator().manual_seed(1000)
+    for p in params:
+        p.grad = (torch.randn(p.shape, generator=ggen) * 1e-2).to(dev)
+    return params, opt
+
+
+def bench_lion(steps, warmup, settle, cpu_baseline, extras):
+    import torch
+
+    dev = "cuda:0"
+    res_small = None
+    if extras:
+        # configuration 3: the GPT-2-small parameter set, 10 steps with fresh seeded gradients each step (copied into the
+        # gradient tensors between the timed steps, outside their events)
+        params, opt = _lion_setup(GPT2_SMALL_SHAPES, dev)
+        n_small = sum(p.numel() for p in params)
+        assert len(params) == 148 and n_small == 124439808
+        fresh = []
+        for s in range(10):
+            gg = torch.Generator().manual_seed(1000 + s)
+            fresh.append((torch.randn(n_small, generator=gg) * 1e-2).to(dev))
+
+        def new_grads(i):
+            at = 0
+            for p in params:
+                p.grad.copy_(fresh[i][at:at + p.numel()].view(p.shape))
+                at += p.numel()
+
+        s_step, s_kernel, s_min, s_info = _time_steps(opt.step, 10, warmup, settle, before_each=new_grads)
+        res_small = {
+            "workload": f"fused Lion step, GPT-2-small set: {len(params)} tensors = {n_small} fp32 params, bf16 momentum, 10 steps with fresh gradients",
+            "ms_per_step": s_step, "kernel_ms_avg": s_kernel, "kernel_ms_min": s_min, "value": 16.0 * n_small / (s_kernel * 1e-3) / 1e9, "unit": "GB/s",
+            "frac": 16.0 * n_small / (s_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": 16.0 * n_small, "settle": s_info,
+            "note": "ms_per_step includes copying the fresh gradients; value and frac are from the events around the step alone",
+        }
+        del opt, params, fresh
+        torch.cuda.empty_cache()
+
+    shapes = LION_LARGE_SHAPES
+    n_params = sum(a * b for a, b in shapes)
+    params, opt = _lion_setup(shapes, dev)
     nbytes = 16.0 * n_params
-    ms_step, ms_kernel, ms_min = _time_steps(opt.step, steps, warmup)
+    ms_step, ms_kernel, ms_min, info = _time_steps(opt.step, steps, warmup, min(settle, 20))
     res = {
-        "value": nbytes / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms_step, "dtype": "f32 params/grads, bf16 momentum",
+        "value": nbytes / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms_step, "dtype": "f32 params/grads, bf16 momentum", "settle": info,
         "roofline": {
             "bound": "hbm", "achieved": nbytes / (ms_kernel * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": nbytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": _measured_traffic("lion"),
+            "frac": nbytes / (ms_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": _measured_traffic("lion"), "traffic_source": TRAFFIC_SOURCE,
             "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "bytes_per_launch": nbytes,
         },
         "workload": f"fused Lion step, {len(shapes)} tensors (39 x 2048x8192 + 39 x 8192x2048) = {n_params} fp32 params, bf16 momentum",
     }
+    if res_small is not None:
+        res["configs"] = {"3_lion_gpt2_small": res_small}
     if cpu_baseline:
         # bounded sample: 8 of the 78 tensors (134,217,728 parameters) through the four reference statements on all host
         # cores, 3 steps
@@ -169,15 +307,15 @@ def bench_lion(steps, warmup, cpu_baseline):
         ps = [params[i].detach().cpu().clone() for i in range(n_t)]
         gs = [params[i].grad.cpu().clone() for i in range(n_t)]
         ms = [opt.state[params[i]]["exp_avg"].cpu().clone() for i in range(n_t)]
-        lion_step_torch(ps, gs, ms, hp["lr"], hp["betas"], hp["weight_decay"])     # warm-up
+        lion_step_torch(ps, gs, ms, LION_HP["lr"], LION_HP["betas"], LION_HP["weight_decay"])     # warm-up
         reps = 3
         t0 = time.perf_counter()
         for _ in range(reps):
-            lion_step_torch(ps, gs, ms, hp["lr"], hp["betas"], hp["weight_decay"])
+            lion_step_torch(ps, gs, ms, LION_HP["lr"], LION_HP["betas"], LION_HP["weight_decay"])
         dt = (time.perf_counter() - t0) / reps
         n_el = sum(p.numel() for p in ps)
         res["cpu_baseline"] = {
-            "value": 16.0 * n_el / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "value": 16.0 * n_el / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "cpu_model": _cpu_model(), "kind": "port",
             "sample": f"{n_t} of 78 tensors ({n_el} parameters), vanilla 4-statement PyTorch Lion step on the host, {dt * 1e3:.1f} ms per step, {reps} steps",
         }
     del opt, params
@@ -188,13 +326,15 @@ def bench_lion(steps, warmup, cpu_baseline):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # defaults: the GPU's clocks take a few dozen launches to settle after idling (per-launch time of the attention
-    # kernel wanders by 25 % over the first 30 launches, then stays within 1 %), so the warm-up is longer than usual
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--settle", type=int, default=100,
+                    help="clock-settle launches ahead of the warm-up of every timed section (reported, not counted as warm-up)")
     ap.add_argument("--path", choices=["both", "attn", "lion", "copy"], default="both",
                     help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the two headline kernels (no backward, library GEMM or other configurations): for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: both kernels are single-device and this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -217,8 +357,9 @@ def main():
         print(json.dumps({"copy_bytes_read": 4 * n, "copy_bytes_written": 4 * n, "launches": args.warmup + args.steps}))
         return
     cpu = not args.no_cpu_baseline
-    attn = bench_attention(args.steps, args.warmup, cpu) if args.path in ("both", "attn") else None
-    lion = bench_lion(args.steps, args.warmup, cpu) if args.path in ("both", "lion") else None
+    extras = not args.headline_only
+    attn = bench_attention(args.steps, args.warmup, args.settle, cpu, extras) if args.path in ("both", "attn") else None
+    lion = bench_lion(args.steps, args.warmup, args.settle, cpu, extras) if args.path in ("both", "lion") else None
     head = attn if attn is not None else lion
     line = {
         "metric": "FA fwd TFLOP/s (bf16, S=8K D=128 causal) + fused Lion HBM GB/s",
@@ -230,15 +371,22 @@ def main():
         "data": "synthetic",
         "config": {"workload": head["workload"] + ("; second path: " + lion["workload"] if attn is not None and lion is not None else "")},
         "roofline": head["roofline"],
+        "settle": head["settle"],
     }
     if "cpu_baseline" in head:
         line["cpu_baseline"] = head["cpu_baseline"]
     if attn is not None and lion is not None:
-        line["lion"] = {k: v for k, v in lion.items() if k != "workload"}
+        line["lion"] = {k: v for k, v in lion.items() if k not in ("workload", "configs")}
     if attn is not None and "bwd" in attn:
         line["attn_bwd"] = attn["bwd"]
     if attn is not None and "library_gemm" in attn:
         line["library_gemm"] = attn["library_gemm"]
+    configs = {}
+    for part in (attn, lion):
+        if part is not None:
+            configs.update(part.get("configs", {}))
+    if configs:
+        line["configs"] = configs
     print(json.dumps(line))
 
 

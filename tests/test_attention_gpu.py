@@ -52,6 +52,17 @@ def kernel_variant(request):
     _lib.tune_set("attn.variant", -1)
 
 
+def _kernel_taken(t_q, t_k, t_v, causal):
+    """The kernel the library launches for these [B, H, S, D] tensors with the current attn.variant (fo_attn_fwd_kernel)."""
+    import ctypes
+
+    I3 = ctypes.c_int64 * 3
+    B, H, Sq, D = t_q.shape
+    code = _lib.load().fo_attn_fwd_kernel(B, H, Sq, t_k.shape[2], D, I3(*t_k.stride()[:3]), I3(*t_v.stride()[:3]), int(causal), 0, 0)
+    assert code >= 0, _lib.strerror(code)
+    return code
+
+
 def _run_and_check(B, H, Sq, Sk, D, dtype, causal, seed=0, scale=None):
     q, k, v = _qkv(B, H, Sq, Sk, D, dtype, seed)
     o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, softmax_scale=scale)
@@ -95,14 +106,64 @@ def test_dtype_causal_headdim_grid(dtype, causal, D):
     _run_and_check(2, 3, 512, 512, D, dtype, causal, seed=3)
 
 
-def test_long_context_slice_of_headline_shape():
-    # the headline shape is B=2 H=16 S=8192 D=128 bf16 causal; two of its (batch, head) slices against the oracle
+@pytest.mark.parametrize("kernel_variant", [0, 16, 32], indirect=True)
+def test_long_context_slice_of_headline_shape(kernel_variant):
+    # the headline shape is B=2 H=16 S=8192 D=128 bf16 causal; two of its (batch, head) slices against the oracle, on each
+    # of the three kernels (so few slices leave the choice to the 128-row kernel; the full shape is tested below)
     _run_and_check(1, 2, 8192, 8192, 128, torch.bfloat16, True, seed=0)
 
 
 def test_throughput_shape_slice_fp16_noncausal():
-    # B=16 H=32 S=2048 D=128 fp16 non-causal; 8 of its (batch, head) slices
+    # B=16 H=32 S=2048 D=128 fp16 non-causal; 8 of its (batch, head) slices (the full shape is tested below)
     _run_and_check(1, 8, 2048, 2048, 128, torch.float16, False, seed=0)
+
+
+def _full_shape_against_oracle(B, H, S, D, dtype, causal, slices, expect_kernel):
+    """The whole benchmark shape through multi_head_attention with the library's own kernel choice (asserted, not
+    assumed), then the listed (batch, head) slices of the result against the oracle."""
+    q, k, v = _qkv(B, H, S, S, D, dtype, seed=0)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    assert _lib.load().fo_tune_get(b"attn.variant") == -1
+    assert _kernel_taken(qd, kd, vd, causal) == expect_kernel, "the benchmark shape does not take the kernel this test is for"
+    o, lse = multi_head_attention(qd, kd, vd, causal=causal, return_lse=True)
+    torch.cuda.synchronize()
+    o, lse = o.cpu(), lse.cpu()
+    worst_o = worst_lse = 0.0
+    for b, h in slices:
+        o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], causal=causal)
+        eo, el = _check(o[b:b + 1, h:h + 1], lse[b:b + 1, h:h + 1], o_ref, lse_ref, f"B{B} H{H} S{S} D{D} {dtype} causal={causal} slice ({b},{h})")
+        worst_o, worst_lse = max(worst_o, eo), max(worst_lse, el)
+    print(f"{len(slices)} slices: max |O err| {worst_o:.3e}, max |LSE err| {worst_lse:.3e}")
+
+
+def test_headline_shape_on_the_kernel_the_benchmark_times():
+    # B=2 H=16 S=8192 D=128 bf16 causal, all 32 (batch, head) slices: 256-row kernel, XCD-mapped workgroup order, 16 items
+    # of two query blocks per head
+    _full_shape_against_oracle(2, 16, 8192, 128, torch.bfloat16, True, [(b, h) for b in range(2) for h in range(16)],
+                               _lib.FO_ATTN_KERNEL_ROWS256_W8)
+
+
+def test_throughput_shape_on_the_kernel_the_benchmark_times():
+    # B=16 H=32 S=2048 D=128 fp16 non-causal (512 heads x 8 items): the first and the last batch element complete and every
+    # fifth slice in between - 154 slices, heads 0..31 and every XCD among them
+    slices = [(b, h) for b in range(16) for h in range(32) if b in (0, 15) or (b * 32 + h) % 5 == 0]
+    assert {(b * 32 + h) % 8 for b, h in slices} == set(range(8)) and max(h for _, h in slices) == 31
+    _full_shape_against_oracle(16, 32, 2048, 128, torch.float16, False, slices, _lib.FO_ATTN_KERNEL_ROWS256_W8)
+
+
+@pytest.mark.parametrize("shape", [(1, 8, 1300, 1300), (2, 8, 800, 1000), (3, 8, 1111, 900), (1, 16, 1537, 1537)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kernel_variant", [16, 32], indirect=True)
+def test_256_row_kernel_with_heads_dealt_to_xcds_and_several_items_per_head(shape, causal, D, kernel_variant):
+    # 8, 16 and 24 heads (a multiple of the 8 XCDs: workgroup id -> (XCD, head, item)) with 3 to 7 items per head, ragged
+    # lengths; causal items are pairs of query blocks, the middle one single when their number is odd
+    if D == 64 and kernel_variant == 32:
+        pytest.skip("head_dim 64 has no four-wave form of the 256-row kernel")
+    B, H, Sq, Sk = shape
+    q, k, v = _qkv(B, H, Sq, Sk, D, torch.bfloat16, seed=Sq + Sk + D)
+    assert _kernel_taken(q, k, v, causal) == kernel_variant
+    _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq + Sk + D)
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 1000), (1, 1, 1000, 64), (3, 5, 191, 191)])
@@ -136,8 +197,18 @@ def test_ragged_across_256_row_blocks_head_dim_64(shape, causal, dtype, kernel_v
     _run_and_check(B, H, Sq, Sk, 64, dtype, causal, seed=Sq + Sk + 64)
 
 
-def test_head_dim_64_large_shape_takes_the_256_row_kernel_by_default():
-    # enough 256-row workgroups for every CU: the library's own choice must agree with the oracle too
+@pytest.mark.parametrize("causal,S", [(True, 2304), (False, 1024)])
+def test_head_dim_64_large_shape_takes_the_256_row_kernel_by_default(causal, S):
+    # enough 256-row workgroups for every CU (80 heads x 5 pairs of query blocks, the middle one single / x 4 blocks), and
+    # more than 2048 queries where causal: the library's own choice is the 256-row kernel, and must agree with the oracle
+    q, k, v = _qkv(2, 40, S, S, 64, torch.bfloat16, seed=5)
+    assert _kernel_taken(q, k, v, causal) == _lib.FO_ATTN_KERNEL_ROWS256_W8
+    _run_and_check(2, 40, S, S, 64, torch.bfloat16, causal, seed=5)
+
+
+def test_causal_up_to_2048_queries_takes_the_128_row_kernel_by_default():
+    q, k, v = _qkv(2, 40, 2048, 2048, 64, torch.bfloat16, seed=5)
+    assert _kernel_taken(q, k, v, True) == _lib.FO_ATTN_KERNEL_ROWS128
     _run_and_check(2, 40, 2048, 2048, 64, torch.bfloat16, True, seed=5)
 
 

@@ -362,21 +362,90 @@ def test_typed_mixed_dtypes_in_one_optimizer_and_state_dict():
         assert _same_bits(params[i].detach().flatten(), exp_p[i]) and _same_bits(st.flatten(), exp_m[i])
     sd = opt.state_dict()
     assert all("exp_avg" in s for s in sd["state"].values())
-    # torch.optim.Optimizer.load_state_dict casts floating-point state to the parameter's dtype (the reference class
-    # inherits the same behaviour); whatever dtype results, the next step must run and agree with the formula
+    # torch.optim.Optimizer.load_state_dict casts floating-point state to the parameter's dtype; this class restores the
+    # dtype each momentum was saved with, so a resumed run continues on the same rounding points
     opt2 = Lion(params, lr=3e-4, betas=(0.95, 0.98), weight_decay=0.01)
     opt2.load_state_dict(sd)
     grads = [(torch.randn(s, generator=g) * 0.01).to(dt) for s, dt in zip(shapes, dts)]
     for i, prm in enumerate(params):
         st2 = opt2.state[prm]["exp_avg"]
-        assert st2.dtype == prm.dtype and torch.equal(st2.float(), opt.state[prm]["exp_avg"].to(prm.dtype).float())
-        exp_m[i] = st2.detach().cpu().flatten().clone()
+        assert st2.dtype == torch.float32 and torch.equal(st2, opt.state[prm]["exp_avg"])
         prm.grad = grads[i].to(DEV)
     opt2.step()
     torch.cuda.synchronize()
     for i, prm in enumerate(params):
         pe, me = lo.lion_step_explicit_typed(exp_p[i], grads[i].flatten(), exp_m[i], 3e-4, (0.95, 0.98), 0.01)
         assert _same_bits(prm.detach().flatten(), pe) and _same_bits(opt2.state[prm]["exp_avg"].flatten(), me)
+
+
+def test_resume_from_a_checkpoint_continues_bit_identically():
+    # fp32 parameters with the default bf16 momentum: 3 steps, checkpoint (through torch.save / torch.load, as a training
+    # script would), 3 more steps on a fresh optimizer - against 6 uninterrupted steps
+    import io
+
+    shapes = [(300, 70), (8192,), (5,)]
+    g = torch.Generator().manual_seed(21)
+    host_p = [torch.randn(s, generator=g) * 0.02 for s in shapes]
+    grads = [[torch.randn(s, generator=g) * 0.01 for s in shapes] for _ in range(6)]
+    hp = dict(lr=1e-3, betas=(0.9, 0.99), weight_decay=0.1)
+
+    def run(params, opt, steps):
+        for it in steps:
+            for prm, gr in zip(params, grads[it]):
+                prm.grad = gr.to(DEV)
+            opt.step()
+
+    straight = [torch.nn.Parameter(t.clone().to(DEV)) for t in host_p]
+    opt_s = Lion(straight, **hp)
+    run(straight, opt_s, range(6))
+    first = [torch.nn.Parameter(t.clone().to(DEV)) for t in host_p]
+    opt_a = Lion(first, **hp)
+    run(first, opt_a, range(3))
+    buf = io.BytesIO()
+    torch.save({"params": [p.detach() for p in first], "opt": opt_a.state_dict()}, buf)
+    buf.seek(0)
+    ckpt = torch.load(buf, weights_only=True)
+    resumed = [torch.nn.Parameter(t.clone()) for t in ckpt["params"]]
+    opt_b = Lion(resumed, **hp)
+    opt_b.load_state_dict(ckpt["opt"])
+    assert all(opt_b.state[p]["exp_avg"].dtype == torch.bfloat16 for p in resumed)
+    run(resumed, opt_b, range(3, 6))
+    torch.cuda.synchronize()
+    for a, b in zip(straight, resumed):
+        assert _same_bits(a.detach().flatten().cpu(), b.detach().flatten().cpu())
+        assert _same_bits(opt_s.state[a]["exp_avg"].flatten().cpu(), opt_b.state[b]["exp_avg"].flatten().cpu())
+
+
+def test_gradients_accumulated_in_place_and_replaced_between_steps():
+    # the step keeps what it learnt about a parameter while its gradient and momentum are the same objects; in-place
+    # changes of the gradient must be seen, a replaced gradient or momentum must be picked up
+    n = 20000
+    g = torch.Generator().manual_seed(4)
+    p0 = torch.randn(n, generator=g) * 0.02
+    gs = [torch.randn(n, generator=g) * 0.01 for _ in range(4)]
+    prm = torch.nn.Parameter(p0.clone().to(DEV))
+    opt = Lion([prm], **HP)
+    pc, mc = p0.numpy().copy(), np.zeros(n, np.uint16)
+    prm.grad = gs[0].to(DEV)
+    opt.step()
+    lo.lion_step_c(pc, gs[0].numpy().copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    prm.grad.copy_(gs[1].to(DEV))                      # same tensor object, new values
+    opt.step()
+    lo.lion_step_c(pc, gs[1].numpy().copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    prm.grad = None                                     # zero_grad(set_to_none=True), then a new gradient tensor
+    keep_alive = torch.empty(n, device=DEV)             # so that the allocator hands out another address
+    prm.grad = gs[2].to(DEV)
+    opt.step()
+    lo.lion_step_c(pc, gs[2].numpy().copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    new_m = (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16)
+    opt.state[prm]["exp_avg"] = new_m.to(DEV)           # momentum replaced by the caller
+    mc = new_m.view(torch.int16).numpy().view(np.uint16).copy()
+    prm.grad.copy_(gs[3].to(DEV))
+    opt.step()
+    lo.lion_step_c(pc, gs[3].numpy().copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    torch.cuda.synchronize()
+    assert np.array_equal(_bits32(prm), pc.view(np.uint32)) and np.array_equal(_bits16(opt.state[prm]["exp_avg"]), mc)
+    del keep_alive
 
 
 def test_typed_unaligned_views_and_multi_tensor_equivalence():
