@@ -323,6 +323,43 @@ def bench_lion(steps, warmup, settle, cpu_baseline, extras):
     return res
 
 
+def bench_clock(steps, warmup, settle):
+    """What the chip's clock does under this kernel: the 256-row attention kernel with 32 ... 512 workgroups (one per CU up
+    to 256, so the launch time is one workgroup's time), the headline shape on random and on all-zero operands, and the
+    vendor library's GEMM on both. Run under `rocprofv3 --pmc GRBM_GUI_ACTIVE --kernel-trace`, the counter divided by a
+    kernel's duration is the clock it ran at."""
+    import torch
+
+    from fast_ops.flash_attention.flash_attention import multi_head_attention
+    from fast_ops_amd import _lib
+
+    dev, S, D = "cuda:0", 8192, 128
+    scale = 1.0 / (D ** 0.5)
+    out = {"busy_cus": [], "operands": [], "gemm": []}
+    (q, k, v), g = _attn_inputs(2, 16, S, D, torch.bfloat16, dev)
+    _lib.tune_set("attn.variant", _lib.FO_ATTN_KERNEL_ROWS256_W8)
+    try:
+        for heads in (2, 4, 8, 12, 16, 32):
+            qq, kk, vv = (t.view(32, S, D)[:heads].view(1, heads, S, D) for t in (q, k, v))
+            _, ms, ms_min, _ = _time_steps(lambda: multi_head_attention(qq, kk, vv, causal=True, softmax_scale=scale), steps, warmup, settle)
+            wgs = heads * 16
+            out["busy_cus"].append({"heads": heads, "workgroups": wgs, "kernel_ms_avg": ms, "kernel_ms_min": ms_min,
+                                    "tflops": 2.0 * heads * S * S * D / (ms * 1e-3) / 1e12})
+        for name, make in (("standard normal", lambda t: t), ("all zero", torch.zeros_like), ("all one", torch.ones_like)):
+            qq, kk, vv = make(q), make(k), make(v)
+            _, ms, ms_min, _ = _time_steps(lambda: multi_head_attention(qq, kk, vv, causal=True, softmax_scale=scale), steps, warmup, settle)
+            out["operands"].append({"operands": name, "kernel_ms_avg": ms, "kernel_ms_min": ms_min, "tflops": 2.0 * 32 * S * S * D / (ms * 1e-3) / 1e12})
+    finally:
+        _lib.tune_set("attn.variant", -1)
+    n = 8192
+    a, b = (torch.randn(n, n, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
+    for name, make in (("standard normal", lambda t: t), ("all zero", torch.zeros_like)):
+        aa, bb = make(a), make(b)
+        _, ms, ms_min, _ = _time_steps(lambda: torch.matmul(aa, bb), steps, warmup, settle)
+        out["gemm"].append({"operands": name, "kernel_ms_avg": ms, "kernel_ms_min": ms_min, "tflops": 2.0 * n ** 3 / (ms * 1e-3) / 1e12})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -330,8 +367,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle", type=int, default=100,
                     help="clock-settle launches ahead of the warm-up of every timed section (reported, not counted as warm-up)")
-    ap.add_argument("--path", choices=["both", "attn", "lion", "copy"], default="both",
-                    help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by")
+    ap.add_argument("--path", choices=["both", "attn", "lion", "copy", "clock"], default="both",
+                    help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
+                         "clock: the attention kernel against the number of busy CUs and the operand bits, with the library GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the two headline kernels (no backward, library GEMM or other configurations): for profiler runs")
@@ -355,6 +393,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": 4 * n, "copy_bytes_written": 4 * n, "launches": args.warmup + args.steps}))
+        return
+    if args.path == "clock":
+        print(json.dumps(bench_clock(args.steps, args.warmup, args.settle)))
         return
     cpu = not args.no_cpu_baseline
     extras = not args.headline_only

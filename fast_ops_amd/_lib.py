@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfastops_hip.so")
 
 FO_LION_CHUNK = 8192
+FO_ATTN_BWD_STATIC_ROWS = 1 << 20
 FO_DTYPE_F16, FO_DTYPE_BF16, FO_DTYPE_F32 = 0, 1, 2
 FO_ATTN_KERNEL_ROWS128, FO_ATTN_KERNEL_ROWS128_EXACT, FO_ATTN_KERNEL_ROWS256_W8, FO_ATTN_KERNEL_ROWS256_W4 = 0, 1, 16, 32
 
@@ -36,6 +37,7 @@ SIGNATURES = {
     "fo_attn_fwd": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [_I64P] * 4 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "fo_attn_fwd_kernel": (ctypes.c_int, [ctypes.c_int] * 5 + [_I64P] * 2 + [ctypes.c_int] * 3),
     "fo_attn_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 5 + [ctypes.POINTER(_I64P), ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "fo_attn_bwd_static_ws": (ctypes.c_int, [ctypes.c_void_p] * 9 + [ctypes.c_int] * 5 + [ctypes.POINTER(_I64P), ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "fo_attn_fwd_dropout": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [_I64P] * 4 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]),
     "fo_dropout_mask": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p]),
     "fo_attn_fwd_ex": (ctypes.c_int, [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [_I64P] * 4 + [ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),

@@ -27,6 +27,8 @@
 // 128-row forward kernel.
 #include <type_traits>
 
+#include <mutex>
+
 #include "attn_common.hpp"
 
 namespace fo {
@@ -998,12 +1000,35 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
 
 using namespace fo;
 
+// ---- the same without a workspace argument and without any allocation: delta lives in a device array of this library.
+// The array's name is only a host-side handle for the device symbol; its address on a device comes from
+// hipGetSymbolAddress, asked once per device with that device current, and only that pointer is handed to the kernels.
+constexpr int64_t kStaticDeltaFloats = FO_ATTN_BWD_STATIC_ROWS;
+static __device__ __align__(256) float scratch[kStaticDeltaFloats];
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[kMaxDevices];   // per device; null until that device's first call
+
+static int scratch_of_current_device(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FO_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return FO_ERR_LAUNCH;
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return FO_OK;
+}
+
 static int attn_bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                          float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
                          const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, float dropout_p,
                          uint32_t seed, uint64_t rng_offset, const void* bias, const int64_t* bias_strides, int bias_dtype,
-                         void* stream) {
-  if (!q || !k || !v || !o || !d_o || !lse || !delta_ws || !dq || !dk || !dv || !strides_host) return FO_ERR_NULL_POINTER;
+                         void* stream, bool static_ws = false) {
+  // static_ws: delta_ws is ignored and the library's own per-device array takes its place (fo_attn_bwd_static_ws)
+  if (!q || !k || !v || !o || !d_o || !lse || (!delta_ws && !static_ws) || !dq || !dk || !dv || !strides_host) return FO_ERR_NULL_POINTER;
   for (int t = 0; t < 8; ++t)
     if (!strides_host[t]) return FO_ERR_NULL_POINTER;
   if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
@@ -1019,7 +1044,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   }
   const uintptr_t all = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv;
   if (all & 15u) return FO_ERR_MISALIGNED;
-  if (((uintptr_t)lse | (uintptr_t)delta_ws) & 3u) return FO_ERR_MISALIGNED;
+  if (((uintptr_t)lse | (static_ws ? 0 : (uintptr_t)delta_ws)) & 3u) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;
   if (!(dropout_p >= 0.0f) || dropout_p >= 1.0f) return FO_ERR_BAD_SHAPE;
   if (bias) {
@@ -1027,6 +1052,12 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
     if (bias_dtype != FO_DTYPE_F32 && bias_dtype != dtype) return FO_ERR_BAD_DTYPE;
     if (bias_strides[0] < 0 || bias_strides[1] < 0 || bias_strides[2] < 0) return FO_ERR_BAD_STRIDE;
     if ((uintptr_t)bias & (bias_dtype == FO_DTYPE_F32 ? 3u : 1u)) return FO_ERR_MISALIGNED;
+  }
+  if (static_ws) {
+    // (after every argument check: a rejected call has made no HIP call)
+    if ((int64_t)B * H * Sq > kStaticDeltaFloats) return FO_ERR_BAD_SHAPE;
+    const int st = scratch_of_current_device(&delta_ws);
+    if (st != FO_OK) return st;
   }
 
   AttnBwdParams p;
@@ -1064,6 +1095,15 @@ extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const vo
                            const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream) {
   return attn_bwd_impl(q, k, v, o, d_o, lse, delta_ws, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
                        0.0f, 0u, 0ull, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int fo_attn_bwd_static_ws(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                                     void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                                     const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream) {
+  // Every delta element the dK/dV kernel reads (rows below Sq of each head) is written by the dQ kernel of the same
+  // call, so what an earlier call left in the array does not matter and nothing has to be cleared.
+  return attn_bwd_impl(q, k, v, o, d_o, lse, nullptr, dq, dk, dv, B, H, Sq, Sk, D, strides_host, softmax_scale, causal, dtype,
+                       0.0f, 0u, 0ull, nullptr, nullptr, 0, stream, true);
 }
 
 extern "C" int fo_attn_bwd_dropout(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,

@@ -116,6 +116,19 @@ int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, cons
                 float* delta_ws, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
                 const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream);
 
+/* fo_attn_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no workspace argument, and the call itself allocates and frees nothing. The
+ * [B, H, Sq] fp32 delta buffer lives in a device array of the library (FO_ATTN_BWD_STATIC_ROWS floats = 4 MiB, which
+ * each GPU the library runs on holds until the process ends). B*H*Sq above FO_ATTN_BWD_STATIC_ROWS is refused with
+ * FO_ERR_BAD_SHAPE. Same results as fo_attn_bwd, bit for bit. All calls on one GPU share the array: calls that
+ * overlap on one GPU (different streams or threads) race on it and must be serialised by the caller; calls in stream
+ * order on one stream are safe. The first call on a device looks up the array's address there (hipGetSymbolAddress;
+ * not while a capture is in progress). No counterpart in the reference. */
+#define FO_ATTN_BWD_STATIC_ROWS (1 << 20)
+int fo_attn_bwd_static_ws(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                          void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk, int D,
+                          const int64_t* const* strides_host, float softmax_scale, int causal, int dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------------
  * The same two with dropout of the attention probabilities, as the reference's Triton kernels define it
  * (flash_attention_triton.py:38-50 hash, :125,:216-219 forward, :421,:524-532,:551,:599 backward): element
