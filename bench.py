@@ -1,7 +1,7 @@
 """Benchmark of the two hot paths on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle N] [--path both|attn|lion|copy] [--no-cpu-baseline]
-                    [--headline-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle N] [--path both|attn|lion|copy|clock|ablations]
+                    [--no-cpu-baseline] [--headline-only]
 
 Prints ONE JSON line. The headline value is the attention forward throughput at B=2 H=16 S=8192 D=128 bf16 causal
 (FLOPs counted as 2*B*H*S^2*D); the fused Lion step over 1,308,622,848 fp32 parameters with bf16 momentum (16 bytes
@@ -360,6 +360,37 @@ def bench_clock(steps, warmup, settle):
     return out
 
 
+def bench_ablations(steps, warmup, settle):
+    """Timing ablations of the 256-row attention kernel at the headline shape: what each part of the kernel costs in
+    cycles and in clock. Needs a library built with `python -m fast_ops_amd.build --ablations` (the variants leave work
+    out and produce wrong results by design; a default build does not contain them). Under
+    `rocprofv3 --pmc GRBM_GUI_ACTIVE SQ_VALU_MFMA_BUSY_CYCLES --kernel-trace` every variant is a kernel of its own name."""
+    import torch
+
+    from fast_ops.flash_attention.flash_attention import multi_head_attention
+    from fast_ops_amd import _lib
+
+    if _lib.load().fo_tune_get(b"build.ablations") != 1:
+        print("bench.py --path ablations needs a library built with `python -m fast_ops_amd.build --ablations`", file=sys.stderr)
+        sys.exit(2)
+    B, H, S, D = 2, 16, 8192, 128
+    (q, k, v), _ = _attn_inputs(B, H, S, D, torch.bfloat16, "cuda:0")
+    scale = 1.0 / (D ** 0.5)
+    names = {16: "full kernel (eight waves x 32 rows)", 257: "no global->LDS copies", 258: "no exponentials (and no scale-and-shift)",
+             260: "no LDS fragment reads", 263: "none of the three", 320: "no barrier", 32: "four waves x 64 rows", 0: "128-row kernel"}
+    out = []
+    try:
+        for causal, variants in ((False, (16, 257, 258, 260, 263, 320, 32)), (True, (16, 32, 0))):
+            flops = (2.0 if causal else 4.0) * B * H * S * S * D
+            for var in variants:
+                _lib.tune_set("attn.variant", var)
+                _, ms, ms_min, _ = _time_steps(lambda: multi_head_attention(q, k, v, causal=causal, softmax_scale=scale), steps, warmup, settle)
+                out.append({"causal": causal, "variant": var, "what": names[var], "kernel_ms_avg": ms, "kernel_ms_min": ms_min, "tflops_equivalent": flops / (ms * 1e-3) / 1e12})
+    finally:
+        _lib.tune_set("attn.variant", -1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -367,9 +398,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle", type=int, default=100,
                     help="clock-settle launches ahead of the warm-up of every timed section (reported, not counted as warm-up)")
-    ap.add_argument("--path", choices=["both", "attn", "lion", "copy", "clock"], default="both",
+    ap.add_argument("--path", choices=["both", "attn", "lion", "copy", "clock", "ablations"], default="both",
                     help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
-                         "clock: the attention kernel against the number of busy CUs and the operand bits, with the library GEMM")
+                         "clock: the attention kernel against the number of busy CUs and the operand bits, with the library GEMM; "
+                         "ablations: the attention kernel with parts left out (needs a build with --ablations)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the two headline kernels (no backward, library GEMM or other configurations): for profiler runs")
@@ -396,6 +428,9 @@ def main():
         return
     if args.path == "clock":
         print(json.dumps(bench_clock(args.steps, args.warmup, args.settle)))
+        return
+    if args.path == "ablations":
+        print(json.dumps(bench_ablations(args.steps, args.warmup, args.settle)))
         return
     cpu = not args.no_cpu_baseline
     extras = not args.headline_only
