@@ -43,6 +43,7 @@ struct AttnBwdParams {
   float* delta;
   void *dq, *dk, *dv;
   int B, H, Sq, Sk;
+  int d;                // true head_dim: a multiple of 8, at most the D the kernels are compiled for
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];   // element strides: batch, head, sequence
   float scale, scale_log2e;
   int head_group;       // heads per group in the order of the workgroups (see bwd_item)
@@ -124,9 +125,9 @@ __device__ __forceinline__ void acc_fence(f32x16 (&acc)[N]) {
 // Copy of a 64-row tile (rows row0 .. row0+63 of a [S, D] matrix with row stride `stride`) into LDS by the whole
 // workgroup: per wave D/32 direct-to-LDS instructions. Each instruction fills 1 KiB of LDS with the 64 lanes' pieces
 // back to back, so the swizzle is applied by choosing which global chunk a lane fetches. Rows past the end re-read
-// the last row (callers mask them).
+// the last row (callers mask them); columns from the true head_dim `d` on read zeros.
 template <typename T, int D>
-__device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int row0, int S, FO_LDS char* dst, int wave_s, int lane_in) {
+__device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int row0, int S, int d, FO_LDS char* dst, int wave_s, int lane_in) {
   // (an opaque copy of the lane index: this is the path of tiles that cross the end of the matrix, taken once per
   // workgroup at most; its address arithmetic must not be hoisted out of it into registers that live across the loop)
   int lane = lane_in;
@@ -140,7 +141,7 @@ __device__ __forceinline__ void copy_tile64(const T* base, int64_t stride, int r
     const int row = (wave_s * DMA_PER_WAVE + i) * ROWS_PER_DMA + lane / CHUNKS;
     const int col = ((lane % CHUNKS) ^ swz<D>(row)) * 8;
     const int r = min(row0 + row, S - 1);
-    dma16_lane_ptr(base + (int64_t)r * stride + col, dst + (wave_s * DMA_PER_WAVE + i) * 1024);
+    dma16_lane_ptr(live_or_zero(base + (int64_t)r * stride + col, col, d), dst + (wave_s * DMA_PER_WAVE + i) * 1024);
   }
 }
 
@@ -151,10 +152,10 @@ template <typename T, int D>
 struct TileLaneOffsets {
   static constexpr int N = kBwdTile * D * 2 / 1024 / kBwdWaves;   // pieces per wave and tile
   uint32_t off[N];
-  bool ok;                                                        // 32-bit offsets suffice for this row stride
-  __device__ __forceinline__ void init(int64_t stride, int wave_s, int lane) {
+  bool ok;                                                        // 32-bit offsets suffice for this row stride, and the rows have all D columns
+  __device__ __forceinline__ void init(int64_t stride, int d, int wave_s, int lane) {
     constexpr int ROW_BYTES = D * 2, CHUNKS = ROW_BYTES / 16, ROWS_PER_DMA = 1024 / ROW_BYTES;
-    ok = stride < (1 << 23);
+    ok = stride < (1 << 23) && d == D;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       const int row = (wave_s * N + i) * ROWS_PER_DMA + lane / CHUNKS;
@@ -195,10 +196,10 @@ __device__ __forceinline__ typename Ops<T>::vec8 col_frag(FO_LDS const char* til
 // 32*db + 8*rg + 4*hh + u) written to memory. Straight from the registers that is 8 bytes per lane to 32 different
 // rows per instruction (4.3 us per workgroup for dK and dV, during which the workgroup's LDS and registers keep the
 // next one waiting); instead the rows are rounded into LDS (`stage`, 32 rows padded by 16 bytes each, this wave's
-// own) and leave as whole 16-byte pieces, 64 lanes covering consecutive rows. Rows from n_rows on are not written.
+// own) and leave as whole 16-byte pieces, 64 lanes covering consecutive rows. Rows from n_rows on and columns from the true head_dim `d` on are not written.
 template <typename T, int D>
 __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], float mul, FO_LDS char* stage, T* base, int64_t stride,
-                                                   int row0, int n_rows, int lane) {
+                                                   int row0, int n_rows, int d, int lane) {
   constexpr int ROW_BYTES = D * 2, OROW = ROW_BYTES + 16, CH = ROW_BYTES / 16;
   typedef __attribute__((ext_vector_type(4))) T vec4;
   typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -216,7 +217,7 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
   for (int it = 0; it < 32 * CH / 64; ++it) {
     const int idx = it * 64 + lane, row = idx / CH, ch = idx % CH;
     const i32x4 piece = *(FO_LDS const i32x4*)(stage + row * OROW + ch * 16);
-    if (row0 + row < n_rows) *(i32x4*)(base + (int64_t)(row0 + row) * stride + ch * 8) = piece;
+    if (row0 + row < n_rows && ch * 8 < d) *(i32x4*)(base + (int64_t)(row0 + row) * stride + ch * 8) = piece;
   }
 }
 constexpr int stage_bytes(int D) { return 32 * (D * 2 + 16); }   // per wave and matrix
@@ -246,8 +247,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   const int n_tiles = CAUSAL ? (min(Sk, q0 + kBwdRows) + kBwdTile - 1) / kBwdTile : (Sk + kBwdTile - 1) / kBwdTile;
 
   TileLaneOffsets<T, D> klo, vlo;
-  klo.init(prm.ks[2], wave_s, lane);
-  vlo.init(prm.vs[2], wave_s, lane);
+  klo.init(prm.ks[2], prm.d, wave_s, lane);
+  vlo.init(prm.vs[2], prm.d, wave_s, lane);
   // A bias that is the same for every query (query stride 0) is 64 values per key tile, the same for all lanes: wave 0
   // copies them into LDS with the tile (4 bytes per lane: one key in fp32, two in the operand type), and every lane
   // reads its registers' keys from there. (Loaded from global memory where they are used, the compiler waits for
@@ -271,8 +272,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
       copy_tile64_inside<T, D>(kbase, prm.ks[2], tile * kBwdTile, klo, smem + buf * TILE_BYTES, wave_s);
       copy_tile64_inside<T, D>(vbase, prm.vs[2], tile * kBwdTile, vlo, smem + (2 + buf) * TILE_BYTES, wave_s);
     } else {
-      copy_tile64<T, D>(kbase, prm.ks[2], tile * kBwdTile, Sk, smem + buf * TILE_BYTES, wave_s, lane);
-      copy_tile64<T, D>(vbase, prm.vs[2], tile * kBwdTile, Sk, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(kbase, prm.ks[2], tile * kBwdTile, Sk, prm.d, smem + buf * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(vbase, prm.vs[2], tile * kBwdTile, Sk, prm.d, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
     }
   };
   issue(0, 0);
@@ -284,7 +285,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     const T* qp = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1] + (int64_t)qrow * prm.qs[2] + 8 * hh;
     const T* gp = (const T*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + (int64_t)qrow * prm.dos[2] + 8 * hh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) { qf[ks] = *(const vec8*)(qp + 16 * ks); gf[ks] = *(const vec8*)(gp + 16 * ks); }
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      qf[ks] = *(const vec8*)live_or_zero(qp + 16 * ks, 16 * ks + 8 * hh, prm.d);
+      gf[ks] = *(const vec8*)live_or_zero(gp + 16 * ks, 16 * ks + 8 * hh, prm.d);
+    }
   }
   const float lse2 = prm.lse[(int64_t)bh * Sq + qrow] * kLog2e;
   // delta_i = sum_d dO_id O_id (flash_attention_triton.py:273-315), negated: this lane holds half of its row's dO
@@ -295,7 +299,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     const T* op = (const T*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)qrow * prm.os[2] + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-      const vec8 ov = *(const vec8*)(op + 16 * ks);
+      const vec8 ov = *(const vec8*)live_or_zero(op + 16 * ks, 16 * ks + 8 * hh, prm.d);
 #pragma unroll
       for (int e = 0; e < 8; ++e) delta -= (float)ov[e] * (float)gf[ks][e];
     }
@@ -437,7 +441,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
         vec4 o4;
 #pragma unroll
         for (int u = 0; u < 4; ++u) o4[u] = (T)(acc[db][rg * 4 + u] * scale);
-        *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
+        if (32 * db + 8 * rg + 4 * hh < prm.d) *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
       }
   }
 }
@@ -467,8 +471,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;   // queries before the block's first key never attend it
 
   TileLaneOffsets<T, D> qlo, glo;
-  qlo.init(prm.qs[2], wave_s, lane);
-  glo.init(prm.dos[2], wave_s, lane);
+  qlo.init(prm.qs[2], prm.d, wave_s, lane);
+  glo.init(prm.dos[2], prm.d, wave_s, lane);
   // ---- bias. A lane owns a key and its registers run over queries, so a bias that is the same for every query (query
   // stride 0) is one value per lane for the whole kernel. Otherwise the wave's 64 queries x 32 keys of a tile are
   // copied straight into LDS together with the tile (a load the compiler can see is waited for right where it is
@@ -513,8 +517,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
       copy_tile64_inside<T, D>(qbase, prm.qs[2], qt * kBwdTile, qlo, smem + buf * TILE_BYTES, wave_s);
       copy_tile64_inside<T, D>(gbase, prm.dos[2], qt * kBwdTile, glo, smem + (2 + buf) * TILE_BYTES, wave_s);
     } else {
-      copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
-      copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, prm.d, smem + buf * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, prm.d, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
     }
     // per-row LSE and delta of the tile, 4 bytes per lane, also straight into LDS (a load the compiler can see would
     // make it wait for the tile copies as well); rows past the end re-read the last row and are masked below
@@ -533,7 +537,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
     const T* kp = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1] + (int64_t)krow * prm.ks[2] + 8 * hh;
     const T* vp = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1] + (int64_t)krow * prm.vs[2] + 8 * hh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) { kf[ks] = *(const vec8*)(kp + 16 * ks); vf[ks] = *(const vec8*)(vp + 16 * ks); }
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      kf[ks] = *(const vec8*)live_or_zero(kp + 16 * ks, 16 * ks + 8 * hh, prm.d);
+      vf[ks] = *(const vec8*)live_or_zero(vp + 16 * ks, 16 * ks + 8 * hh, prm.d);
+    }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(kf[ks]), "v"(vf[ks]));
   }
@@ -660,8 +667,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
   {
     FO_LDS char* stage = smem + wave_s * stage_bytes(D);
     const int k0w_s = k0 + wave_s * 32;
-    store_rows_via_lds<T, D>(dkacc, scale, stage, (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1], prm.dks[2], k0w_s, Sk, lane);
-    store_rows_via_lds<T, D>(dvacc, 1.0f, stage, (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1], prm.dvs[2], k0w_s, Sk, lane);
+    store_rows_via_lds<T, D>(dkacc, scale, stage, (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1], prm.dks[2], k0w_s, Sk, prm.d, lane);
+    store_rows_via_lds<T, D>(dvacc, 1.0f, stage, (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1], prm.dvs[2], k0w_s, Sk, prm.d, lane);
   }
 }
 
@@ -703,15 +710,15 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   const int ja = CAUSAL ? min(k0w / kBwdTile, n_qt) : 0;     // ... and this wave's keys start later still
 
   TileLaneOffsets<T, D> qlo, glo;
-  qlo.init(prm.qs[2], wave_s, lane);
-  glo.init(prm.dos[2], wave_s, lane);
+  qlo.init(prm.qs[2], prm.d, wave_s, lane);
+  glo.init(prm.dos[2], prm.d, wave_s, lane);
   auto issue = [&](int qt, int buf) {
     if (qt * kBwdTile + kBwdTile <= Sq && qlo.ok && glo.ok) {
       copy_tile64_inside<T, D>(qbase, prm.qs[2], qt * kBwdTile, qlo, smem + buf * TILE_BYTES, wave_s);
       copy_tile64_inside<T, D>(gbase, prm.dos[2], qt * kBwdTile, glo, smem + (NBUF + buf) * TILE_BYTES, wave_s);
     } else {
-      copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, smem + buf * TILE_BYTES, wave_s, lane);
-      copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, smem + (NBUF + buf) * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(qbase, prm.qs[2], qt * kBwdTile, Sq, prm.d, smem + buf * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(gbase, prm.dos[2], qt * kBwdTile, Sq, prm.d, smem + (NBUF + buf) * TILE_BYTES, wave_s, lane);
     }
     if (wave_s < 2) {
       const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
@@ -740,8 +747,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     const T* vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      copy_tile64<T, D>(kbase, prm.ks[2], k0 + 64 * half, Sk, smem + (1 + half) * TILE_BYTES, wave_s, lane);
-      copy_tile64<T, D>(vbase, prm.vs[2], k0 + 64 * half, Sk, smem + (NBUF + 1 + half) * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(kbase, prm.ks[2], k0 + 64 * half, Sk, prm.d, smem + (1 + half) * TILE_BYTES, wave_s, lane);
+      copy_tile64<T, D>(vbase, prm.vs[2], k0 + 64 * half, Sk, prm.d, smem + (NBUF + 1 + half) * TILE_BYTES, wave_s, lane);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
@@ -953,8 +960,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   {
     FO_LDS char* stage = smem + wave_s * stage_bytes(D);
     const int k0w_s = k0 + wave_s * 32;
-    store_rows_via_lds<T, D>(dkacc, scale, stage, (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1], prm.dks[2], k0w_s, Sk, lane);
-    store_rows_via_lds<T, D>(dvacc, 1.0f, stage, (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1], prm.dvs[2], k0w_s, Sk, lane);
+    store_rows_via_lds<T, D>(dkacc, scale, stage, (T*)prm.dk + b * prm.dks[0] + h * prm.dks[1], prm.dks[2], k0w_s, Sk, prm.d, lane);
+    store_rows_via_lds<T, D>(dvacc, 1.0f, stage, (T*)prm.dv + b * prm.dvs[0] + h * prm.dvs[1], prm.dvs[2], k0w_s, Sk, prm.d, lane);
   }
 }
 
@@ -991,7 +998,8 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   // (delta is computed by the dQ kernel, which the dK/dV kernel follows)
   attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(q);
   // attn_bwd.variant 0 selects the plain dK/dV kernel everywhere (tests compare the two)
-  if (!DROP && !BIAS && tune(g_attn_bwd_variant) != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(q);
+  // (and every head_dim other than the two the kernels are compiled for)
+  if (!DROP && !BIAS && p.d == D && tune(g_attn_bwd_variant) != 0) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(q);
   else attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(q);
   return launch_status();
 }
@@ -1032,7 +1040,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   for (int t = 0; t < 8; ++t)
     if (!strides_host[t]) return FO_ERR_NULL_POINTER;
   if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
-  if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
+  if (D < 8 || D > 128 || D % 8 != 0) return FO_ERR_BAD_HEAD_DIM;
   if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || (int64_t)B * H * Sq > (1ll << 40)) return FO_ERR_BAD_SHAPE;
   for (int t = 0; t < 8; ++t) {
     // rows start on 16-byte boundaries (8 elements); only the inputs K and V may repeat a head (stride 0 = multi-query)
@@ -1062,7 +1070,7 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
 
   AttnBwdParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse; p.delta = delta_ws; p.dq = dq; p.dk = dk; p.dv = dv;
-  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.d = D;
   int64_t* dst[8] = {p.qs, p.ks, p.vs, p.os, p.dos, p.dqs, p.dks, p.dvs};
   for (int t = 0; t < 8; ++t)
     for (int i = 0; i < 3; ++i) dst[t][i] = strides_host[t][i];
@@ -1084,8 +1092,9 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
 #define FO_BWD2(T, DD, BI) (drop ? (c ? launch_bwd<T, DD, true, true, BI>(p, s) : launch_bwd<T, DD, false, true, BI>(p, s)) \
                                  : (c ? launch_bwd<T, DD, true, false, BI>(p, s) : launch_bwd<T, DD, false, false, BI>(p, s)))
 #define FO_BWD(T, DD) (bias ? FO_BWD2(T, DD, true) : FO_BWD2(T, DD, false))
-  if (dtype == FO_DTYPE_BF16) return D == 128 ? FO_BWD(__bf16, 128) : FO_BWD(__bf16, 64);
-  return D == 128 ? FO_BWD(_Float16, 128) : FO_BWD(_Float16, 64);
+  // kernels are compiled for 64 and 128 columns; a head_dim in between runs on the next one with zero columns
+  if (dtype == FO_DTYPE_BF16) return D > 64 ? FO_BWD(__bf16, 128) : FO_BWD(__bf16, 64);
+  return D > 64 ? FO_BWD(_Float16, 128) : FO_BWD(_Float16, 64);
 #undef FO_BWD
 #undef FO_BWD2
 }

@@ -48,6 +48,16 @@ __device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst
 #endif
 }
 
+// Sixteen zero bytes in device memory. A head_dim below the 64 or 128 columns a kernel is compiled for is handled by
+// addresses alone: whatever would read columns past the true head_dim - a lane's piece of a tile copy, a fragment
+// loaded from a row - reads these zeros instead, so the padded columns of every operand are zero (they add nothing to a
+// product) and nothing is read past the end of a row; stores of such columns are skipped.
+static __device__ __attribute__((aligned(16))) const uint32_t kZero16[4] = {0u, 0u, 0u, 0u};
+template <typename T>
+__device__ __forceinline__ const T* live_or_zero(const T* ptr, int col, int d) {
+  return col < d ? ptr : (const T*)kZero16;
+}
+
 // Dropout of attention probabilities, as the reference defines it (flash_attention_triton.py:38-50,125,216-219): element
 // (b*H + h, q, key) has the 32-bit index  offset + (b*H + h)*Sq*Sk + q*Sk + key  (all arithmetic modulo 2^32); the index,
 // xored with the seed, goes through an integer hash, and the element is KEPT iff the hash exceeds

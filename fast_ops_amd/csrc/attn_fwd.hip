@@ -39,6 +39,7 @@ constexpr int kBN = 64;            // keys per tile
 struct AttnParams {
   const void* q; const void* k; const void* v; void* o; float* lse;
   int B, H, Sq, Sk;
+  int d;                                // true head_dim: a multiple of 8, at most the D the kernel is compiled for (128-row kernel only)
   int64_t qs[3], ks[3], vs[3], os[3];   // element strides: batch, head, sequence
   float scale_log2e;                    // softmax_scale * log2(e)
   int n_qblk;
@@ -132,7 +133,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const int key0 = tile * kBN;
     FO_LDS char* kdst = smem + buf * TILE_BYTES;
     FO_LDS char* vdst = smem + (2 + buf) * TILE_BYTES;
-    if (key0 + kBN <= Sk) {
+    if (key0 + kBN <= Sk && prm.d == D) {
       const char* ktile = (const char*)(kbase + (int64_t)key0 * prm.ks[2]);
       const char* vtile = (const char*)(vbase + (int64_t)key0 * prm.vs[2]);
 #pragma unroll
@@ -144,7 +145,8 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     } else {
       // last, partial tile: rows past the end re-read the last key (masked later). Runs at most once per workgroup;
       // the opaque copy of the lane id keeps its address arithmetic from being hoisted out of the tile loop, where
-      // it would hold registers for the whole kernel.
+      // it would hold registers for the whole kernel. Also every tile of a head_dim below D: columns from the true
+      // head_dim on read zeros.
       int lane_here = lane;
       asm volatile("" : "+v"(lane_here));
 #pragma unroll
@@ -153,8 +155,8 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
         const int col = ((lane_here % CHUNKS) ^ swz<D>(row)) * 8;
         const int key = min(key0 + row, Sk - 1);
         const int lds_off = (wave_s * DMA_PER_WAVE + i) * 1024;
-        dma16_lane_ptr(kbase + (int64_t)key * prm.ks[2] + col, kdst + lds_off);
-        dma16_lane_ptr(vbase + (int64_t)key * prm.vs[2] + col, vdst + lds_off);
+        dma16_lane_ptr(live_or_zero(kbase + (int64_t)key * prm.ks[2] + col, col, prm.d), kdst + lds_off);
+        dma16_lane_ptr(live_or_zero(vbase + (int64_t)key * prm.vs[2] + col, col, prm.d), vdst + lds_off);
       }
     }
   };
@@ -195,7 +197,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const int qrow = min(q0w + l32, Sq - 1);
     const T* qp = qbase + (int64_t)qrow * prm.qs[2] + 8 * hh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *(const vec8*)(qp + 16 * ks);
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *(const vec8*)live_or_zero(qp + 16 * ks, 16 * ks + 8 * hh, prm.d);
     // Consume the fragments here so that the compiler waits for these loads before the loop instead of inside it:
     // a vmcnt wait inside the loop would also wait for the direct-to-LDS copies in flight, which it does not see.
 #pragma unroll
@@ -430,7 +432,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
         vec4 o4;
 #pragma unroll
         for (int j = 0; j < 4; ++j) o4[j] = (T)(oacc[db][rg * 4 + j] * inv);
-        *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
+        if (32 * db + 8 * rg + 4 * hh < prm.d) *(vec4*)(op + 32 * db + 8 * rg + 4 * hh) = o4;
       }
     if (prm.lse != nullptr && hh == 0) {
       // ln sum_j exp(scale*s_j) = ln2 * (m*scale*log2e + log2(l))
@@ -1085,8 +1087,8 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 // `forced` is the value of attn.variant (-1: the library's choice). Values from 256 on are timing ablations and exist
 // only in a build with FO_ABLATIONS.
 static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, int forced) {
-  // dropout and bias run on the 128-row kernel
-  if (p.bias.ptr != nullptr || dropout) return FO_ATTN_KERNEL_ROWS128;
+  // dropout, bias and head dims other than 64 and 128 run on the 128-row kernel
+  if (p.bias.ptr != nullptr || dropout || p.d != D) return FO_ATTN_KERNEL_ROWS128;
   // The 256-row kernel addresses a head's keys with 32-bit byte offsets ...
   const bool wide_ok = (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
   // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
@@ -1162,7 +1164,7 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
                          const void* bias, const int64_t* bias_strides, int bias_dtype, void* stream) {
   if (!q || !k || !v || !o || !qs || !ks || !vs || !os) return FO_ERR_NULL_POINTER;
   if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
-  if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
+  if (D < 8 || D > 128 || D % 8 != 0) return FO_ERR_BAD_HEAD_DIM;
   if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return FO_ERR_BAD_SHAPE;
   const int64_t n_qblk = ((int64_t)Sq + kBM - 1) / kBM;
   if (n_qblk * B * H > 0x7FFFFFFFll || (int64_t)B * H * Sq > (1ll << 40)) return FO_ERR_BAD_SHAPE;
@@ -1192,7 +1194,7 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
 
   AttnParams p;
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
-  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.d = D;
   for (int i = 0; i < 3; ++i) { p.qs[i] = qs[i]; p.ks[i] = ks[i]; p.vs[i] = vs[i]; p.os[i] = os[i]; }
   p.scale_log2e = softmax_scale * 1.4426950408889634f;
   p.n_qblk = (int)n_qblk;
@@ -1210,21 +1212,22 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
                     (p.bias.strides[1] * elt) % 16 == 0 && (p.bias.strides[2] * elt) % 16 == 0;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == FO_DTYPE_BF16) return D == 128 ? launch<__bf16, 128>(p, causal != 0, drop, s) : launch<__bf16, 64>(p, causal != 0, drop, s);
-  return D == 128 ? launch<_Float16, 128>(p, causal != 0, drop, s) : launch<_Float16, 64>(p, causal != 0, drop, s);
+  // kernels are compiled for 64 and 128 columns; a head_dim in between runs on the next one with zero columns
+  if (dtype == FO_DTYPE_BF16) return D > 64 ? launch<__bf16, 128>(p, causal != 0, drop, s) : launch<__bf16, 64>(p, causal != 0, drop, s);
+  return D > 64 ? launch<_Float16, 128>(p, causal != 0, drop, s) : launch<_Float16, 64>(p, causal != 0, drop, s);
 }
 
 extern "C" int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* ks, const int64_t* vs,
                                   int causal, int has_bias, int has_dropout) {
   if (!ks || !vs) return FO_ERR_NULL_POINTER;
-  if (D != 64 && D != 128) return FO_ERR_BAD_HEAD_DIM;
+  if (D < 8 || D > 128 || D % 8 != 0) return FO_ERR_BAD_HEAD_DIM;
   if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return FO_ERR_BAD_SHAPE;
   if (ks[2] < D || vs[2] < D || ks[2] >= kMaxRowStride || vs[2] >= kMaxRowStride) return FO_ERR_BAD_STRIDE;
   AttnParams p = {};
-  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.d = D;
   for (int i = 0; i < 3; ++i) { p.ks[i] = ks[i]; p.vs[i] = vs[i]; }
   p.bias.ptr = has_bias ? (const void*)ks : nullptr;   // (only tested against NULL)
-  return choose_kernel(p, D, causal != 0, has_dropout != 0, tune(g_attn_variant));
+  return choose_kernel(p, D > 64 ? 128 : 64, causal != 0, has_dropout != 0, tune(g_attn_variant));
 }
 
 extern "C" int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,

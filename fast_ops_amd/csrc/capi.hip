@@ -16,7 +16,7 @@ extern "C" const char* fo_strerror(int status) {
     case FO_OK: return "ok";
     case FO_ERR_NULL_POINTER: return "a required pointer is NULL";
     case FO_ERR_BAD_DTYPE: return "unsupported dtype: inputs must be half-precision floating point (float16 or bfloat16)";
-    case FO_ERR_BAD_HEAD_DIM: return "unsupported head_dim: this build implements head_dim 64 and 128";
+    case FO_ERR_BAD_HEAD_DIM: return "unsupported head_dim: it must be a multiple of 8 from 8 to 128";
     case FO_ERR_BAD_SHAPE: return "a size is not positive or is too large";
     case FO_ERR_BAD_STRIDE: return "bad stride: rows must be contiguous in head_dim and start on 16-byte boundaries";
     case FO_ERR_MISALIGNED: return "a base pointer is not aligned as required";

@@ -130,16 +130,6 @@ def attn_fwd_strided(
     if D % 8 != 0:
         raise RuntimeError("head_dim must be a multiple of 8")                        # flash_attention.py:65-66
     scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(D)             # flash_attention_triton.py:750
-    if D not in (64, 128):
-        # The kernels exist for head_dim 64 and 128. Any other multiple of 8 (the reference's contract,
-        # flash_attention.py:61-66) runs on zero-padded copies: padded columns add nothing to Q K^T, and the padded
-        # columns of V only produce output columns that are dropped; the scale stays that of the true head_dim.
-        Dp = 64 if D < 64 else 128
-        pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
-        o_p, lse = attn_fwd_strided(pad(q), pad(k), pad(v), dims, causal, scale, dropout, bias)
-        o = torch.empty_like(q)
-        o.copy_(o_p.narrow(id_, 0, D))
-        return o, lse
     o = torch.empty_like(q)
     if o.stride() != q.stride():   # empty_like keeps dense layouts; anything else gets a plain contiguous output
         o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
@@ -175,12 +165,6 @@ def attn_bwd_strided(
     scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(D)
     if d_o.dtype != q.dtype or d_o.shape != q.shape:
         raise RuntimeError(f"dO must have the output's shape and dtype, got {tuple(d_o.shape)} {d_o.dtype}")
-    if D not in (64, 128):
-        # same zero padding as the forward; O's padded columns are zero, so delta and the padded gradient columns are too
-        Dp = 64 if D < 64 else 128
-        pad = lambda t: torch.nn.functional.pad(t, (0, Dp - D))
-        dq, dk, dv = attn_bwd_strided(pad(q), pad(k), pad(v), pad(o), lse, pad(d_o), dims, causal, scale, dropout, bias)
-        return tuple(t.narrow(id_, 0, D).contiguous() for t in (dq, dk, dv))
     if d_o.stride(-1) != 1 or any(s % 8 for s in d_o.stride()[:-1]):
         d_o = d_o.contiguous()
     if o.stride(-1) != 1:
@@ -278,8 +262,7 @@ def multi_head_attention(
 ) -> Union[Tensor, Tuple[Tensor, Tensor]]:
     """FlashAttention forward (https://arxiv.org/abs/2205.14135), B = batch, H = heads, M = queries, N = keys, D = head dim.
 
-    Limitations (violations raise RuntimeError): head_dim a multiple of 8 up to 128 (64 and 128 run in place, the others
-    on zero-padded copies); the last dimension of Q, K, V contiguous and rows 16-byte aligned; inputs float16 or
+    Limitations (violations raise RuntimeError): head_dim a multiple of 8 up to 128; the last dimension of Q, K, V contiguous and rows 16-byte aligned; inputs float16 or
     bfloat16; GPU tensors.
 
     :param Q: (B, H, M, D) Query tensor.

@@ -26,8 +26,8 @@ typedef enum fo_status {
   FO_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
   FO_ERR_BAD_DTYPE = -2,      /* dtype code is not FO_DTYPE_F16 / FO_DTYPE_BF16 (the reference dispatches half types only,
                                  flash_attention/common/launch_utils.h:8-21) */
-  FO_ERR_BAD_HEAD_DIM = -3,   /* head_dim not supported (reference contract: <= 128 and a multiple of 8,
-                                 flash_attention.py:61-66; this library implements 64 and 128) */
+  FO_ERR_BAD_HEAD_DIM = -3,   /* head_dim not supported: the reference's contract, a multiple of 8 up to 128
+                                 (flash_attention.py:61-66), is what this library implements */
   FO_ERR_BAD_SHAPE = -4,      /* a size is <= 0, or too large for the kernel's indexing */
   FO_ERR_BAD_STRIDE = -5,     /* a stride breaks the layout contract (rows must be 16-byte aligned) */
   FO_ERR_MISALIGNED = -6,     /* a base pointer is not aligned as required */
@@ -71,7 +71,9 @@ int fo_tune_get(const char* key);
  *   causal       non-zero: query i attends keys j <= i (top-left aligned, attention_ref.py:54-58)
  *   dtype        FO_DTYPE_F16 or FO_DTYPE_BF16, for q, k, v and o alike
  *
- * Requirements checked here: D in {64, 128}; Sq, Sk >= 1; softmax_scale finite and > 0; base pointers and row strides
+ * Requirements checked here: D a multiple of 8 from 8 to 128 (64 and 128 are the sizes the kernels are laid out for; any
+ * other runs on the next of the two with the missing columns read as zeros and never stored - no copies, the same
+ * results, the speed of the larger size); Sq, Sk >= 1; softmax_scale finite and > 0; base pointers and row strides
  * multiples of 16 bytes; sequence strides of k and v below 2^24 elements (FO_ERR_BAD_STRIDE otherwise: the kernels
  * address the rows of a key tile with 32-bit byte offsets).
  */
@@ -109,7 +111,7 @@ int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* k_str
  *   dq / dk, dv         [B, H, Sq, D] / [B, H, Sk, D], written for every element; never read
  *   strides_host        eight pointers to three element strides each (batch, head, sequence; head_dim stride 1), in
  *                       the order q, k, v, o, d_o, dq, dk, dv. Only the inputs may repeat a batch or head (stride 0).
- * Same requirements as fo_attn_fwd (D in {64, 128}, 16-byte aligned pointers and rows, scale finite and > 0).
+ * Same requirements as fo_attn_fwd (D a multiple of 8 up to 128, 16-byte aligned pointers and rows, scale finite and > 0).
  * Two launches on `stream`; no atomics, results are deterministic.
  */
 int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,

@@ -126,8 +126,9 @@ def test_config2_gpt2_small_shape_slice():
     _run(2, 12, 1024, 1024, 64, torch.bfloat16, True, seed=2)
 
 
-@pytest.mark.parametrize("D", [8, 40, 96])
-def test_other_head_dims_by_padding(D):
+@pytest.mark.parametrize("D", [8, 16, 24, 32, 40, 48, 56, 72, 80, 88, 96, 104, 112, 120])
+def test_every_other_head_dim_of_the_reference_contract(D):
+    # any multiple of 8 up to 128 (flash_attention.py:61-66), inside the kernels: no padded copies
     _run(1, 2, 150, 210, D, torch.float16, True, seed=D)
     _run(1, 2, 97, 97, D, torch.bfloat16, False, seed=D + 1, scale=0.3)
 
@@ -179,3 +180,58 @@ def test_gradients_are_deterministic():
         o = FlashAttentionFunction.apply(qd, kd, vd, True)
         outs.append(torch.autograd.grad(o, (qd, kd, vd), go.to(DEV)))
     assert all(torch.equal(a, b) for a, b in zip(*outs))
+
+
+@pytest.mark.parametrize("D,row", [(40, 48), (8, 16), (104, 128), (56, 64)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_columns_past_the_head_dim_are_neither_read_nor_written(D, row, causal):
+    """Operands and results as views of wider tensors (row stride `row` > head_dim D) whose extra columns hold NaN: a
+    kernel that read a column past D would turn its results into NaN, one that wrote there would overwrite the NaN."""
+    B, H, Sq, Sk = 2, 3, 150, 210
+    q, k, v, go = _inputs(B, H, Sq, Sk, D, torch.bfloat16, seed=D + row)
+    sc = 1.0 / math.sqrt(D)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal, softmax_scale=sc)
+    pt = _half_precision_torch(q, k, v, go, causal, sc)
+
+    def wide(t):
+        w = torch.full(t.shape[:-1] + (row,), float("nan"), dtype=t.dtype, device=DEV)
+        w[..., :D] = t.to(DEV)
+        return w
+
+    qw, kw, vw, gw = wide(q), wide(k), wide(v), wide(go)
+    from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided, attn_fwd_strided
+    o, lse = attn_fwd_strided(qw[..., :D], kw[..., :D], vw[..., :D], (0, 1, 2, 3), causal, sc)
+    assert bool(torch.isfinite(o.float()).all()) and bool(torch.isfinite(lse).all())
+    from oracle.attention_oracle import attention_fwd_oracle
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, softmax_scale=sc)
+    assert float((o.float().cpu() - o_ref).abs().max()) <= 2e-2 and float((lse.cpu() - lse_ref).abs().max()) <= 1e-3
+    ow = wide(o.cpu())
+    got = attn_bwd_strided(qw[..., :D], kw[..., :D], vw[..., :D], ow[..., :D], lse, gw[..., :D], (0, 1, 2, 3), causal, sc)
+    torch.cuda.synchronize()
+    _check(got, ref, pt, f"D{D} in rows of {row} causal={causal}")
+    # results written into views of wider buffers through the C ABI: the columns past D keep their contents
+    import ctypes
+    from fast_ops_amd import _lib
+    I3 = ctypes.c_int64 * 3
+    P64 = ctypes.POINTER(ctypes.c_int64)
+    outs = [torch.full(t.shape[:-1] + (row,), 7.0, dtype=torch.bfloat16, device=DEV) for t in (q, k, v)]
+    o_out = torch.full(q.shape[:-1] + (row,), 7.0, dtype=torch.bfloat16, device=DEV)
+    lse2 = torch.empty(B, H, Sq, dtype=torch.float32, device=DEV)
+    st = lambda t: I3(*t.stride()[:3])
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = _lib.load().fo_attn_fwd(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), o_out.data_ptr(), lse2.data_ptr(), B, H, Sq, Sk, D,
+                                 st(qw), st(kw), st(vw), st(o_out), sc, int(causal), _lib.FO_DTYPE_BF16, stream)
+    assert rc == 0, _lib.strerror(rc)
+    delta = torch.empty(B, H, Sq, dtype=torch.float32, device=DEV)
+    tensors = (qw, kw, vw, ow, gw, outs[0], outs[1], outs[2])
+    arrays = [st(t) for t in tensors]
+    strides = (P64 * 8)(*[ctypes.cast(a, P64) for a in arrays])
+    rc = _lib.load().fo_attn_bwd(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), ow.data_ptr(), gw.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                                 outs[0].data_ptr(), outs[1].data_ptr(), outs[2].data_ptr(), B, H, Sq, Sk, D, strides, sc, int(causal),
+                                 _lib.FO_DTYPE_BF16, stream)
+    assert rc == 0, _lib.strerror(rc)
+    torch.cuda.synchronize()
+    assert torch.equal(o_out[..., :D], o)
+    for w, g_ in zip(outs + [o_out], list(got) + [o]):
+        assert torch.equal(w[..., :D], g_)
+        assert bool((w[..., D:] == 7.0).all()), "a column past the head_dim was written"

@@ -239,10 +239,11 @@ def test_moving_row_maximum(pattern, causal, D, dtype, kernel_variant):
     _check(o, lse, o_ref, lse_ref, f"{pattern} D{D} {dtype} causal={causal}")
 
 
-@pytest.mark.parametrize("D", [8, 16, 24, 32, 40, 72, 96, 104, 120])
+@pytest.mark.parametrize("D", [8, 16, 24, 32, 40, 48, 56, 72, 80, 88, 96, 104, 112, 120])
 @pytest.mark.parametrize("causal", [False, True])
 def test_every_head_dim_of_the_reference_contract(D, causal):
-    # head_dim any multiple of 8 up to 128 (flash_attention.py:61-66); default scale is 1/sqrt(true head_dim)
+    # head_dim any multiple of 8 up to 128 (flash_attention.py:61-66), inside the kernels (no padded copies); default
+    # scale is 1/sqrt(true head_dim)
     _run_and_check(2, 3, 150, 210, D, torch.float16, causal, seed=D)
     _run_and_check(1, 2, 97, 97, D, torch.bfloat16, causal, seed=D + 1, scale=0.3)
 

@@ -58,7 +58,7 @@ def test_attn_argument_validation_without_device():
     assert call(q=None) == -1
     assert call(qs=None) == -1
     assert call(dtype=2) == -2
-    assert call(D=72) == -3
+    assert call(D=68) == -3 and call(D=0) == -3 and call(D=136) == -3      # multiples of 8 from 8 to 128 only
     assert call(D=256) == -3
     assert call(Sq=0) == -4
     assert call(B=-1) == -4
@@ -81,7 +81,7 @@ def test_attn_backward_bias_dropout_argument_validation_without_device():
         1, 1, kw.get("Sq", 128), 128, kw.get("D", 64), kw.get("strides", strides()), kw.get("scale", 0.125), 0, kw.get("dtype", 1), None)
     assert bwd(q=None) == -1 and bwd(ws=None) == -1 and bwd(strides=None) == -1
     assert bwd(dtype=2) == -2
-    assert bwd(D=96) == -3
+    assert bwd(D=100) == -3 and bwd(D=136) == -3
     assert bwd(Sq=0) == -4 and bwd(scale=0.0) == -4
     assert bwd(strides=strides(I3(128 * 64, 64 * 128, 60))) == -5      # dQ rows not 16-byte aligned / shorter than D
     assert bwd(lse=0x1002) == -6
@@ -190,7 +190,9 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
         assert k(1, 1, 512, 512, 64, 1) == _lib.FO_ATTN_KERNEL_ROWS128_EXACT
     finally:
         lib.fo_tune_set(b"attn.variant", -1)
-    assert k(1, 1, 128, 128, 72, 0) == -3 and k(0, 1, 128, 128, 64, 0) == -4
+    assert k(1, 1, 128, 128, 76, 0) == -3 and k(0, 1, 128, 128, 64, 0) == -4
+    # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
+    assert k(2, 16, 8192, 8192, 96, 1) == _lib.FO_ATTN_KERNEL_ROWS128
     assert lib.fo_attn_fwd_kernel(1, 1, 128, 128, 64, None, dense(128, 64), 0, 0, 0) == -1
     # K/V row strides of 2^24 elements and more do not fit the kernels' 32-bit tile offsets: rejected, not wrapped
     wide_rows = I3(0, 0, 1 << 24)
