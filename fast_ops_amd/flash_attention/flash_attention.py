@@ -26,6 +26,8 @@ from torch.autograd import Function
 from .. import _lib
 
 _DTYPE_CODE = {torch.float16: _lib.FO_DTYPE_F16, torch.bfloat16: _lib.FO_DTYPE_BF16}
+# the raw hipStream_t that is current on a device, without building a torch.cuda.Stream object around it
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (lambda dev: torch.cuda.current_stream(dev).cuda_stream)
 _I64x3 = ctypes.c_int64 * 3
 
 
@@ -112,13 +114,20 @@ def dropout_mask(
     return keep.view(torch.bool)
 
 
-def attn_fwd_strided(
-    q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int], causal: bool, softmax_scale: Optional[float],
-    dropout: Optional[Dropout] = None, bias: Optional[Tensor] = None,
-) -> Tuple[Tensor, Tensor]:
-    """Launches fo_attn_fwd (fo_attn_fwd_dropout when ``dropout`` is given, fo_attn_fwd_ex when ``bias`` is). ``dims`` =
-    positions of (batch, head, sequence, head_dim) in the tensors' shapes; ``bias`` is [B|1, H|1, Sq|1, Sk] whatever
-    ``dims`` says. Returns (O with q's shape, dtype and layout; LSE fp32 [B, H, Sq])."""
+class _FwdPlan:
+    """What a forward call of one (shapes, strides, dtype, device, layout) needs besides the data pointers: checked once,
+    then reused - the checks, the stride arrays for the C ABI and the sizes cost more host time than a small kernel runs."""
+    __slots__ = ("B", "H", "Sq", "Sk", "D", "qs", "ks", "vs", "os", "o_dense_like_q", "dtype_code", "device_index", "lse_shape")
+
+
+_FWD_PLANS: dict = {}
+
+
+def _fwd_plan(q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int]) -> _FwdPlan:
+    key = (q.shape, q.stride(), k.shape, k.stride(), v.shape, v.stride(), q.dtype, k.dtype, v.dtype, q.device, k.device, v.device, dims)
+    plan = _FWD_PLANS.get(key)
+    if plan is not None:
+        return plan
     _check_inputs(q, k, v)
     ib, ih, is_, id_ = dims
     B, H, Sq, D = q.shape[ib], q.shape[ih], q.shape[is_], q.shape[id_]
@@ -129,26 +138,59 @@ def attn_fwd_strided(
         raise RuntimeError("FlashAttention only support head dimensions up to 128")  # flash_attention_triton.py:745
     if D % 8 != 0:
         raise RuntimeError("head_dim must be a multiple of 8")                        # flash_attention.py:65-66
-    scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(D)             # flash_attention_triton.py:750
-    o = torch.empty_like(q)
-    if o.stride() != q.stride():   # empty_like keeps dense layouts; anything else gets a plain contiguous output
-        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    plan = _FwdPlan()
+    plan.B, plan.H, plan.Sq, plan.Sk, plan.D = B, H, Sq, Sk, D
     strides = lambda t: _I64x3(t.stride(ib), t.stride(ih), t.stride(is_))
+    plan.qs, plan.ks, plan.vs = strides(q), strides(k), strides(v)
+    o = torch.empty_like(q)
+    plan.o_dense_like_q = o.stride() == q.stride()    # empty_like keeps dense layouts; anything else gets a plain contiguous output
+    if not plan.o_dense_like_q:
+        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    plan.os = strides(o)
+    plan.dtype_code = _DTYPE_CODE[q.dtype]
+    plan.device_index = q.device.index if q.device.index is not None else torch.cuda.current_device()
+    plan.lse_shape = (B, H, Sq)
+    if len(_FWD_PLANS) > 4096:
+        _FWD_PLANS.clear()
+    _FWD_PLANS[key] = plan
+    return plan
+
+
+def attn_fwd_strided(
+    q: Tensor, k: Tensor, v: Tensor, dims: Tuple[int, int, int, int], causal: bool, softmax_scale: Optional[float],
+    dropout: Optional[Dropout] = None, bias: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """Launches fo_attn_fwd (fo_attn_fwd_dropout when ``dropout`` is given, fo_attn_fwd_ex when ``bias`` is). ``dims`` =
+    positions of (batch, head, sequence, head_dim) in the tensors' shapes; ``bias`` is [B|1, H|1, Sq|1, Sk] whatever
+    ``dims`` says. Returns (O with q's shape, dtype and layout; LSE fp32 [B, H, Sq])."""
+    plan = _fwd_plan(q, k, v, dims)
+    scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(plan.D)        # flash_attention_triton.py:750
+    o = torch.empty_like(q) if plan.o_dense_like_q else torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty(plan.lse_shape, dtype=torch.float32, device=q.device)
     if bias is not None:
-        bias = _expand_bias(bias, q, B, H, Sq, Sk)
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream(q.device).cuda_stream
+        bias = _expand_bias(bias, q, plan.B, plan.H, plan.Sq, plan.Sk)
+    dev = plan.device_index
+    lib = _lib.load()
+    # (the launch goes to the stream that is current on the tensors' device; the device is made current only when it is not)
+    guard = torch.cuda.device(dev) if torch.cuda.current_device() != dev else None
+    if guard is not None:
+        guard.__enter__()
+    try:
+        stream = _raw_stream(dev)
         args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
-                B, H, Sq, Sk, D, strides(q), strides(k), strides(v), strides(o),
-                scale, int(bool(causal)), _DTYPE_CODE[q.dtype])
+                plan.B, plan.H, plan.Sq, plan.Sk, plan.D, plan.qs, plan.ks, plan.vs, plan.os,
+                scale, 1 if causal else 0, plan.dtype_code)
         if bias is not None:
-            status = _lib.load().fo_attn_fwd_ex(*args, ctypes.byref(_extras(bias, dropout)), stream)
+            status = lib.fo_attn_fwd_ex(*args, ctypes.byref(_extras(bias, dropout)), stream)
         elif dropout is None or dropout[0] == 0.0:
-            status = _lib.load().fo_attn_fwd(*args, stream)
+            status = lib.fo_attn_fwd(*args, stream)
         else:
-            status = _lib.load().fo_attn_fwd_dropout(*args, float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64), stream)
-    _lib.check(status, "fo_attn_fwd")
+            status = lib.fo_attn_fwd_dropout(*args, float(dropout[0]), dropout[1] & 0xFFFFFFFF, dropout[2] % (1 << 64), stream)
+    finally:
+        if guard is not None:
+            guard.__exit__(None, None, None)
+    if status != 0:
+        _lib.check(status, "fo_attn_fwd")
     return o, lse
 
 
@@ -275,7 +317,11 @@ def multi_head_attention(
     :param dropout_state: (seed, offset) of the mask; default: taken from torch's generator, which is advanced
     :returns: (B, H, M, D)
     """
-    drop = _dropout_arg(dropout_p, dropout_state, Q.shape[0] * Q.shape[1] * Q.shape[2] * K.shape[2])
+    drop = None if dropout_p == 0.0 else _dropout_arg(dropout_p, dropout_state, Q.shape[0] * Q.shape[1] * Q.shape[2] * K.shape[2])
+    if not (torch.is_grad_enabled() and (Q.requires_grad or K.requires_grad or V.requires_grad)):
+        # nothing to differentiate: no autograd node (its bookkeeping costs more host time than a small kernel runs)
+        o, lse = attn_fwd_strided(Q, K, V, (0, 1, 2, 3), causal, softmax_scale, drop)
+        return (o, lse) if return_lse else o
     return FlashAttentionFunction.apply(Q, K, V, causal, softmax_scale, return_lse, drop)
 
 
@@ -287,5 +333,8 @@ def flash_attn(
     differentiable in q, k and v, with dropout and with an additive bias on the scaled scores: [B|1, H|1, 1, seqlen_k]
     or [B|1, H|1, seqlen_q, seqlen_k], the dtype of q or fp32 (:752-768). A bias that requires grad makes the backward
     raise, as in the reference (:854)."""
-    drop = _dropout_arg(dropout_p, dropout_state, q.shape[0] * q.shape[2] * q.shape[1] * k.shape[1])
+    drop = None if dropout_p == 0.0 else _dropout_arg(dropout_p, dropout_state, q.shape[0] * q.shape[2] * q.shape[1] * k.shape[1])
+    if not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad or (bias is not None and bias.requires_grad))):
+        o, lse = attn_fwd_strided(q, k, v, (0, 2, 1, 3), causal, softmax_scale, drop, bias)
+        return (o, lse) if return_lse else o
     return _FlashAttnBSHD.apply(q, k, v, causal, softmax_scale, return_lse, drop, bias)
