@@ -180,8 +180,10 @@ class Lion(Optimizer):
                 if grad is None:
                     continue
                 rec = seen.get(param)
-                if rec is not None and rec[0] is grad and rec[1] is self.state[param].get("exp_avg"):
-                    # same gradient and momentum objects as last step (gradients accumulated in place)
+                if (rec is not None and rec[0] is grad and rec[1] is self.state[param].get("exp_avg")
+                        and rec[3][0] == param.data_ptr() and rec[3][1] == grad.data_ptr() and rec[3][2] == rec[1].data_ptr()):
+                    # same gradient and momentum objects over the same memory as last step (gradients accumulated in
+                    # place): dtypes, devices and layouts cannot have changed, the checks need not be repeated
                     bucket, entry = rec[2], rec[3]
                 else:
                     state = self.state[param]
@@ -233,9 +235,10 @@ class _Table:
             self._copied.synchronize()          # the previous copy out of the staging buffer
         if self._pinned is None or self._pinned.numel() < n:
             self._pinned = torch.empty(max(n, 1), dtype=torch.uint8, pin_memory=True)
-            self.dev = torch.empty(max(n, 1), dtype=torch.uint8, device=self.device)
         self._pinned[:n].numpy()[:] = raw
-        # (the kernel of an earlier step that reads the old table is ahead of this copy on the same stream)
+        # a new device tensor per rebuild: a kernel of an earlier step may still be reading the old table (its memory
+        # goes back to torch's allocator, which hands it out again in stream order)
+        self.dev = torch.empty(max(n, 1), dtype=torch.uint8, device=self.device)
         self.dev[:n].copy_(self._pinned[:n], non_blocking=True)
         if self._copied is None:
             self._copied = torch.cuda.Event()

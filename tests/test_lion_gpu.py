@@ -443,8 +443,13 @@ def test_gradients_accumulated_in_place_and_replaced_between_steps():
     prm.grad.copy_(gs[3].to(DEV))
     opt.step()
     lo.lion_step_c(pc, gs[3].numpy().copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    old_storage = prm.data
+    prm.data = prm.data.clone()                          # the parameter moved to other memory; gradient and momentum objects stay
+    opt.step()
+    lo.lion_step_c(pc, gs[3].numpy().copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
     torch.cuda.synchronize()
     assert np.array_equal(_bits32(prm), pc.view(np.uint32)) and np.array_equal(_bits16(opt.state[prm]["exp_avg"]), mc)
+    assert not torch.equal(old_storage, prm.data)       # the step went to the new memory, not to the old one
     del keep_alive
 
 
