@@ -35,7 +35,13 @@ def dropout_keep_mask(dropout_p: float, seed: int, rng_offset: int, B: int, H: i
     [B, H, M, N], True = kept. Index of (b, h, m, n) = rng_offset + (b*H + h)*M*N + m*N + n in 32-bit arithmetic;
     a = index ^ seed;  a ^= a >> 4;  a = (a ^ 0xDEADBEEF) + (a << 5);  a ^= a >> 11;  keep = a > uint32(fp32(p) * fp32(2^32 - 1)).
     Pinned by tests/test_oracle_attention.py: a pure-Python-integer restatement on small shapes, hand-computed hashes,
-    the kept fraction, and independence of offset-shifted masks."""
+    the kept fraction, and independence of offset-shifted masks.
+    PARITY UNPINNED for one step: the threshold. The reference computes it inside a Triton kernel as
+    ``(dropout_p * 4294967295).to(tl.uint32)`` (flash_attention_triton.py:50); that the product is taken in fp32 (so
+    that the constant becomes 2^32 and the threshold is trunc(fp32(p) * 2^32)) is an inference about the promotion
+    rules of triton 2.0.0.dev20221202, which is not available here, and the reference holds no mask vectors. A double
+    or integer product would move the threshold by at most 2^32 * 2^-24 = 256 of 2^32 hash values: one element in 16
+    million would flip."""
     idx = (np.arange(B * H * M * N, dtype=np.uint64) + np.uint64(rng_offset % (1 << 32))).astype(np.uint32)
     a = idx ^ np.uint32(seed & 0xFFFFFFFF)
     a = a ^ (a >> np.uint32(4))
