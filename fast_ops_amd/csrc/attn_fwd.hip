@@ -477,6 +477,26 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 #ifndef FO_MFMA_NOPS
 #define FO_MFMA_NOPS 1
 #endif
+// Three layout choices of the 256-row kernel, each a bit mask over QB (1: eight waves x 32 rows, 2: four waves x 64 rows),
+// kept as macros so that a build can measure them against each other:
+// FO_PIN_MFMA  the MFMA of a micro-group is fenced to be its first instruction. A lone wave per SIMD issues in order: left
+//              to the compiler, the MFMAs of two neighbouring groups end up back to back with all the other work after
+//              them, and the second one stalls the wave for the 28 cycles the matrix pipe is still busy. Four-wave form:
+//              -6 % cycles; eight-wave form +3 % (its second wave fills such gaps anyway).
+// FO_SPREAD    the copies of a tile are issued one at a time between the MFMAs of its two steps instead of in one batch
+//              behind the tile's barrier, where every wave of the workgroup queues up at the memory pipe at once (a
+//              batch of 8 costs a lone wave ~390 cycles, spread ~110). Four-wave form -10 % cycles on top of the
+//              pinning, eight-wave form -6 %, and the waves reach the barrier closer together (barrier 10 % -> 2.5 %).
+// FO_STAGGER   eight-wave form without FO_SPREAD: the two waves of a SIMD issue the copies of both in turn (-4 % cycles).
+#ifndef FO_PIN_MFMA
+#define FO_PIN_MFMA 2
+#endif
+#ifndef FO_STAGGER
+#define FO_STAGGER 0
+#endif
+#ifndef FO_SPREAD
+#define FO_SPREAD 3
+#endif
 template <typename T, bool NOP> struct AsmMfma;
 #if defined(__HIP_DEVICE_COMPILE__)
 #define FO_MFMA_BODY(PRE, MNEMONIC)                                                                                     \
@@ -552,6 +572,10 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   constexpr int BLOCKS = TILE_BYTES / 1024;      // 1 KiB copy blocks per tile
   constexpr int DMA_PER_WAVE = BLOCKS / kWideWaves;
   static_assert(VFRAGS == KSTEPS && DMA_PER_WAVE >= 1 && KSTEPS >= 4, "tile shape");
+  // Who issues the copies of a tile: every wave its own blocks (ISSUERS == 1), or the two waves of a SIMD in turn, each
+  // the blocks of both (ISSUERS == 2: while one wave is held up at the memory pipe the other has the SIMD to itself).
+  constexpr int ISSUERS = (FO_STAGGER && QB == 1 && !(FO_SPREAD & QB)) ? 2 : 1;
+  constexpr int NBLK = DMA_PER_WAVE * ISSUERS;          // blocks a wave copies per matrix when it is its turn
 
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   FO_LDS char* smem = (FO_LDS char*)smem_raw;    // K ring (kRing tiles) | V ring (kRing tiles)
@@ -632,6 +656,13 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   const int v_lane_row = 8 * (lane >> 5) + 4 * (v_m >> 4) + ((v_m & 7) >> 1), v_lane_col = 16 * ((v_m >> 3) & 1) + 8 * (v_m & 1);
   const uint32_t k_off = (uint32_t)(k_lane_row * (int)prm.ks[2] + k_lane_col) * 2u;
   const uint32_t v_off = (uint32_t)(v_lane_row * (int)prm.vs[2] + v_lane_col) * 2u;
+  // block i of this wave's duty: its own DMA_PER_WAVE blocks, then (ISSUERS == 2) those of the other wave of its SIMD
+  auto blk_of = [&](int i) -> int {
+    if constexpr (ISSUERS == 1) return wave_s * DMA_PER_WAVE + i;
+    else return ((wave_s & 3) + 4 * (i / DMA_PER_WAVE)) * DMA_PER_WAVE + i % DMA_PER_WAVE;
+  };
+  // batch t is this wave's to issue
+  auto my_turn = [&](int t) -> bool { return ISSUERS == 1 || ((t + 4) & 1) == (wave_s >> 2); };
   // one tile of K (ring 0) or V (ring 1) into slot tile % kRing
   auto issue = [&](auto is_v, int tile) {
     constexpr bool V = decltype(is_v)::value;
@@ -640,8 +671,8 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     const int key0 = tile * kBN;
     FO_LDS char* dst = smem + (kRing * (V ? 1 : 0) + (tile & (kRing - 1))) * TILE_BYTES;
 #pragma unroll
-    for (int i = 0; i < DMA_PER_WAVE; ++i) {
-      const int blk = wave_s * DMA_PER_WAVE + i;
+    for (int i = 0; i < NBLK; ++i) {
+      const int blk = blk_of(i);
       const int hf = blk / (BLOCKS / 2), in_half = blk % (BLOCKS / 2);
       // first row (in the tile) and first column of the block
       const int row0 = V ? 32 * hf + 16 * (in_half / DBLK) : 32 * hf + 16 * (in_half & 1);
@@ -662,11 +693,11 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   };
   // The common case, both tiles complete: this wave's blocks have fixed places inside a tile (pointers for tile 0
   // are loop-invariant scalars), and the tile's distance from tile 0 is added to the per-lane offset.
-  const char* k_src0[DMA_PER_WAVE];
-  const char* v_src0[DMA_PER_WAVE];
+  const char* k_src0[NBLK];
+  const char* v_src0[NBLK];
 #pragma unroll
-  for (int i = 0; i < DMA_PER_WAVE; ++i) {
-    const int blk = wave_s * DMA_PER_WAVE + i;
+  for (int i = 0; i < NBLK; ++i) {
+    const int blk = blk_of(i);
     const int hf = blk / (BLOCKS / 2), in_half = blk % (BLOCKS / 2);
     k_src0[i] = (const char*)(kbase + (int64_t)(32 * hf + 16 * (in_half & 1)) * prm.ks[2] + 32 * (in_half >> 1));
     v_src0[i] = (const char*)(vbase + (int64_t)(32 * hf + 16 * (in_half / DBLK)) * prm.vs[2] + 32 * (in_half % DBLK));
@@ -675,20 +706,21 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   const int n_full = min(n_tiles, Sk / kBN);          // tiles below this one are complete
   // batch(t), issued at the top of tile t: K(t+3) and V(t+2). Returns the number of copies this lane issued.
   auto issue_batch = [&](int t) -> int {
+    if (!my_turn(t)) return 0;
     if (t + 3 < n_full && t + 2 >= 0) {
       const uint32_t ko = k_off + (uint32_t)(t + 3) * k_tile_bytes, vo = v_off + (uint32_t)(t + 2) * v_tile_bytes;
-      FO_LDS char* kdst = smem + ((t + 3) & (kRing - 1)) * TILE_BYTES + wave_s * DMA_PER_WAVE * 1024;
-      FO_LDS char* vdst = smem + (kRing + ((t + 2) & (kRing - 1))) * TILE_BYTES + wave_s * DMA_PER_WAVE * 1024;
+      FO_LDS char* kdst = smem + ((t + 3) & (kRing - 1)) * TILE_BYTES;
+      FO_LDS char* vdst = smem + (kRing + ((t + 2) & (kRing - 1))) * TILE_BYTES;
 #pragma unroll
-      for (int i = 0; i < DMA_PER_WAVE; ++i) {
-        dma16_uniform_base(k_src0[i], ko, kdst + i * 1024);
-        dma16_uniform_base(v_src0[i], vo, vdst + i * 1024);
+      for (int i = 0; i < NBLK; ++i) {
+        dma16_uniform_base(k_src0[i], ko, kdst + blk_of(i) * 1024);
+        dma16_uniform_base(v_src0[i], vo, vdst + blk_of(i) * 1024);
       }
-      return 2 * DMA_PER_WAVE;
+      return 2 * NBLK;
     }
     int n = 0;
-    if (t + 3 < n_tiles && t + 3 >= 0) { issue(std::false_type{}, t + 3); n += DMA_PER_WAVE; }
-    if (t + 2 < n_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2); n += DMA_PER_WAVE; }
+    if (t + 3 < n_tiles && t + 3 >= 0) { issue(std::false_type{}, t + 3); n += NBLK; }
+    if (t + 2 < n_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2); n += NBLK; }
     return n;
   };
   issue_batch(-3);
@@ -710,7 +742,9 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       for (int r = 0; r < 16; ++r) oacc[i][qb][r] = 0.0f;
   f32x16 S[2][QB];             // scores: sub-tile s, query block qb live in S[s & 1][qb]
   i32x4 PF[2][QB][2];          // P of sub-tile s: PF[s & 1][qb][16-key step]
-  constexpr bool SPREAD_DMA = (DBG & 8) != 0;   // issue the copies of a tile between the MFMAs of its steps instead of at its top
+  // issue the copies of a tile between the MFMAs of its steps instead of at its top (in the loop of unmasked tiles whose
+  // copies are all whole tiles; everywhere else they go out at the top)
+  constexpr bool SPREAD_DMA = (DBG & 8) != 0 || (FO_SPREAD & QB) != 0;
   constexpr int RD = QB == 2 ? 4 : 2;       // must divide the number of fragments of a sub-tile
   static_assert(KSTEPS % RD == 0, "fragment ring");
   i32x4 KF[RD], VF[RD];        // LDS fragment rings, refilled RD fragments ahead of use
@@ -747,7 +781,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // m = -inf); only then (rarely) the step's P is recomputed from the still intact scores against the true maximum,
   // and O and l are rescaled. The result is that of the exact recurrence (flash_attention_triton.py:200-213,241-243)
   // up to rounding.
-  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop, int dma_tile, auto... no_recovery) {
+  auto step = [&](int s_in, auto parity, auto has_qk, auto has_pv, auto masked, auto in_loop, auto spread, int dma_tile, auto... no_recovery) {
     // (an extra argument: the caller knows that no P of this step can be large, and the recovery path is left out)
     constexpr bool CAN_RECOVER = sizeof...(no_recovery) == 0;
     // inside the loops the MFMAs go without wait states in front unless the build asked for them (see above)
@@ -776,6 +810,15 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     float mc[QB], psum[QB];
 #pragma unroll
     for (int b2 = 0; b2 < QB; ++b2) { mc[b2] = m_run[b2] * c; psum[b2] = 0.0f; }
+    // copies this step issues between its MFMAs (spread): the K blocks of tile dma_tile in the step of an even sub-tile,
+    // the V blocks in that of an odd one
+    constexpr bool SPREAD_HERE = decltype(spread)::value && HAS_QK && HAS_PV;
+    uint32_t dma_off = 0;
+    FO_LDS char* dma_dst = smem;
+    if constexpr (SPREAD_HERE) {
+      dma_off = (P == 0) ? k_off + (uint32_t)dma_tile * k_tile_bytes : v_off + (uint32_t)dma_tile * v_tile_bytes;
+      dma_dst = smem + ((P == 0 ? 0 : kRing) + (dma_tile & (kRing - 1))) * TILE_BYTES + wave_s * DMA_PER_WAVE * 1024;
+    }
     float ex[NEL];
     // score e of NEL: query block, accumulator register (the first 8 registers of every block first: they are the
     // first 16-key step of P V)
@@ -791,25 +834,22 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       } else if (is_qk) {
         if (f == 0) Mfma::v_init_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
         else Mfma::v_acc_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
+        if (FO_PIN_MFMA & QB) __builtin_amdgcn_sched_barrier(0);
         if (qb == QB - 1 && !(DBG & 4)) KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb1, f + RD) : k_frag(kb2, f + RD - KSTEPS);
       } else {
         Mfma::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[P ^ 1][qb][f / DBLK]);
+        if (FO_PIN_MFMA & QB) __builtin_amdgcn_sched_barrier(0);
         if (qb == QB - 1 && !(DBG & 4)) VF[f % RD] = (f + RD < VFRAGS) ? v_frag(vb0, f + RD) : v_frag(vb1, f + RD - VFRAGS);
       }
       if constexpr (!HAS_PV) {
         if (g < RD) VF[g] = v_frag(vb1, g);   // first step: the next one expects the first V^T fragments of sub-tile s
       }
       // -- this group's share of the tile copies (steps of even sub-tiles carry K, of odd ones V)
-      if constexpr (SPREAD_DMA && HAS_QK && HAS_PV) {
+      if constexpr (SPREAD_HERE) {
         constexpr int SPACING = (G - 2) / DMA_PER_WAVE;
         if (g >= 2 && (g - 2) % SPACING == 0 && (g - 2) / SPACING < DMA_PER_WAVE) {
           const int i = (g - 2) / SPACING;
-          if (dma_tile >= 0) {
-            if (P == 0) dma16_uniform_base(k_src0[i], k_off + (uint32_t)dma_tile * k_tile_bytes,
-                                           smem + (dma_tile & (kRing - 1)) * TILE_BYTES + (wave_s * DMA_PER_WAVE + i) * 1024);
-            else dma16_uniform_base(v_src0[i], v_off + (uint32_t)dma_tile * v_tile_bytes,
-                                    smem + (kRing + (dma_tile & (kRing - 1))) * TILE_BYTES + (wave_s * DMA_PER_WAVE + i) * 1024);
-          }
+          dma16_uniform_base(P == 0 ? k_src0[i] : v_src0[i], dma_off, dma_dst + i * 1024);
         }
       }
       // -- this group's share of the softmax arithmetic
@@ -900,10 +940,11 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // ---- tile loop. Tile j runs the steps of sub-tiles 2j and 2j+1; they read K(j), K(j+1), V(j-1), V(j).
   // At its top, copy batches up to (j-2) must have landed - K(j+1) and V(j) are among them - while batch (j-1) may still
   // be in flight; after the barrier every wave is done with tile j-1, so batch j may overwrite K(j-1) and V(j-2).
-  auto tile_top = [&](int j) -> bool {
+  auto tile_top = [&](int j, bool spread_this = false) -> bool {
     if (!(DBG & 32)) {
-      if (__builtin_expect(last_batch == 2 * DMA_PER_WAVE, 1)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_PER_WAVE) : "memory");
-      else if (last_batch >= DMA_PER_WAVE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DMA_PER_WAVE) : "memory");
+      // (as many copies may stay in flight as this wave issued in the batch before: 0, one matrix's or both)
+      if (__builtin_expect(last_batch == 2 * NBLK, 1)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NBLK) : "memory");
+      else if (last_batch >= NBLK) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NBLK) : "memory");
       else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     // A bare barrier: __syncthreads() would first wait for every LDS read in flight, i.e. drain the fragment rings once
@@ -911,7 +952,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     // overwrites, and copies are made visible by the vmcnt wait above (it covers this wave's own pieces; the barrier
     // extends that to everyone's).
     if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
-    if (SPREAD_DMA && j + 3 < n_full) { last_batch = 2 * DMA_PER_WAVE; return true; }   // the steps of this tile issue them
+    if (spread_this) { last_batch = 2 * DMA_PER_WAVE; return true; }   // the steps of this tile issue them
     last_batch = (DBG & 1) ? 0 : issue_batch(j);
     return false;
   };
@@ -958,29 +999,36 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : S[0][b2][r]);
     m_run[b2] = fmaxf(mloc, half_swap(mloc));
   }
-  step(0, P0{}, Y{}, N{}, Y{}, N{}, -1, N{});   // (its reference is its own row maximum: every P <= 1)
-  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, -1);
+  step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1, N{});   // (its reference is its own row maximum: every P <= 1)
+  if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, N{}, -1);
   // Should the steps above have parked registers in scratch memory (they do not at present), wait here, visibly to
   // the compiler, for any reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0)
   // wait that executes on every iteration and also drains the copies in flight, which it does not see.
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), nothing else
   last_batch = (DBG & 1) ? 0 : issue_batch(0);
   int j = 1;
+  if constexpr (SPREAD_DMA) {
+    // unmasked tiles whose copies (K three tiles, V two tiles ahead) are whole tiles: the steps issue them
+    for (; j < min(min(j_mask, n_w - 1), n_full - 3); ++j) {
+      tile_top(j, true);
+      step(2 * j, P0{}, Y{}, Y{}, N{}, Y{}, Y{}, j + 3);
+      step(2 * j + 1, P1{}, Y{}, Y{}, N{}, Y{}, Y{}, j + 2);
+    }
+  }
   for (; j < min(j_mask, n_w - 1); ++j) {
-    const bool sp = tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, N{}, Y{}, sp ? j + 3 : -1);
-    step(2 * j + 1, P1{}, Y{}, Y{}, N{}, Y{}, sp ? j + 2 : -1);
+    tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, N{}, Y{}, N{}, -1);
+    step(2 * j + 1, P1{}, Y{}, Y{}, N{}, Y{}, N{}, -1);
   }
   for (; j < n_w - 1; ++j) {
-    const bool sp = tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, Y{}, Y{}, sp ? j + 3 : -1);
-    step(2 * j + 1, P1{}, Y{}, Y{}, Y{}, Y{}, sp ? j + 2 : -1);
+    tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, Y{}, Y{}, N{}, -1);
+    step(2 * j + 1, P1{}, Y{}, Y{}, Y{}, Y{}, N{}, -1);
   }
   if (j < n_w) {
-    const bool sp = tile_top(j);
-    step(2 * j, P0{}, Y{}, Y{}, Y{}, N{}, sp ? j + 3 : -1);
-    step(2 * j + 1, P1{}, N{}, Y{}, Y{}, N{}, -1);
-    if (sp) issue(std::true_type{}, j + 2);
+    tile_top(j);
+    step(2 * j, P0{}, Y{}, Y{}, Y{}, N{}, N{}, -1);
+    step(2 * j + 1, P1{}, N{}, Y{}, Y{}, N{}, N{}, -1);
     ++j;
   }
   {
@@ -995,8 +1043,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     }
   }
   // tiles in which this wave has nothing to do (causal): keep feeding the workgroup's rings
-  for (; j < n_tiles; ++j)
-    if (tile_top(j)) { issue(std::false_type{}, j + 3); issue(std::true_type{}, j + 2); }
+  for (; j < n_tiles; ++j) tile_top(j);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (CAUSAL && pass + 1 < n_pass) load_q(item);   // (the second pass works on query block `item`)
 
@@ -1097,7 +1144,17 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
   const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
   // (causal, up to 2048 queries: a 256-row block is a large part of the triangle, and the 128-row kernel with its finer
   // blocks, heaviest first, is 10-20 % faster at 1024 queries and equal or a few per cent faster at 2048)
-  int v = forced < 0 ? (wide_ok && wide_wgs >= n_cu && !(causal && p.Sq <= 2048) ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128) : forced;
+  int v = forced;
+  if (forced < 0) {
+    v = (wide_ok && wide_wgs >= n_cu && !(causal && p.Sq <= 2048)) ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128;
+    // head_dim 128 with many key tiles per query block: four waves x 64 rows. Every K / V^T fragment read from LDS feeds two
+    // MFMAs, which costs less energy (at full load the chip's clock is what its power budget leaves) but more cycles per
+    // tile, and its longer pipeline fill and drain have to be spread over enough tiles. Measured on one box, new form
+    // against the eight-wave form: non-causal 2048 keys -1.0 %, 4096 -2.3 %, 8192 -2.5 %; causal 3072 +3 %, 4096 +1 %,
+    // 8192 -0.7 %, 16384 -1.8 %.
+    const int keys = causal ? (p.Sq < p.Sk ? p.Sq : p.Sk) : p.Sk;
+    if (v == FO_ATTN_KERNEL_ROWS256_W8 && D == 128 && keys >= (causal ? 6144 : 2048)) v = FO_ATTN_KERNEL_ROWS256_W4;
+  }
   if (v >= 256) return v;
   if (!wide_ok && v >= 16) v = FO_ATTN_KERNEL_ROWS128;
   if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128) v = FO_ATTN_KERNEL_ROWS128;   // the four-wave form exists for head_dim 128 only
@@ -1130,6 +1187,10 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
         case 256 + 64: return launch_wide<T, D, false, 1, 64>(p, stream);
         case 256 + 128: return launch_wide<T, D, false, 1, 128>(p, stream);
         case 512 + 128: return launch_wide<T, D, false, 2, 128>(p, stream);
+        case 512 + 1: return launch_wide<T, D, false, 2, 1>(p, stream);
+        case 512 + 2: return launch_wide<T, D, false, 2, 2>(p, stream);
+        case 512 + 4: return launch_wide<T, D, false, 2, 4>(p, stream);
+        case 512 + 64: return launch_wide<T, D, false, 2, 64>(p, stream);
         case 512 + 7: return launch_wide<T, D, false, 2, 7>(p, stream);
         case 512 + 8: return launch_wide<T, D, false, 2, 8>(p, stream);
         default: return FO_ERR_UNSUPPORTED;

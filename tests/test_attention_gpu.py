@@ -137,10 +137,10 @@ def _full_shape_against_oracle(B, H, S, D, dtype, causal, slices, expect_kernel)
 
 
 def test_headline_shape_on_the_kernel_the_benchmark_times():
-    # B=2 H=16 S=8192 D=128 bf16 causal, all 32 (batch, head) slices: 256-row kernel, XCD-mapped workgroup order, 16 items
-    # of two query blocks per head
+    # B=2 H=16 S=8192 D=128 bf16 causal, all 32 (batch, head) slices: 256-row kernel (four waves x 64 rows at this length),
+    # XCD-mapped workgroup order, 16 items of two query blocks per head
     _full_shape_against_oracle(2, 16, 8192, 128, torch.bfloat16, True, [(b, h) for b in range(2) for h in range(16)],
-                               _lib.FO_ATTN_KERNEL_ROWS256_W8)
+                               _lib.FO_ATTN_KERNEL_ROWS256_W4)
 
 
 def test_throughput_shape_on_the_kernel_the_benchmark_times():
@@ -148,7 +148,27 @@ def test_throughput_shape_on_the_kernel_the_benchmark_times():
     # fifth slice in between - 154 slices, heads 0..31 and every XCD among them
     slices = [(b, h) for b in range(16) for h in range(32) if b in (0, 15) or (b * 32 + h) % 5 == 0]
     assert {(b * 32 + h) % 8 for b, h in slices} == set(range(8)) and max(h for _, h in slices) == 31
-    _full_shape_against_oracle(16, 32, 2048, 128, torch.float16, False, slices, _lib.FO_ATTN_KERNEL_ROWS256_W8)
+    _full_shape_against_oracle(16, 32, 2048, 128, torch.float16, False, slices, _lib.FO_ATTN_KERNEL_ROWS256_W4)
+
+
+def test_mid_length_causal_shape_takes_the_eight_wave_form_by_default():
+    # B=2 H=16 S=4096 D=128 bf16 causal: long enough for the 256-row kernel, too short for its four-wave form
+    _full_shape_against_oracle(2, 16, 4096, 128, torch.bfloat16, True, [(b, h) for b in range(2) for h in range(16)],
+                               _lib.FO_ATTN_KERNEL_ROWS256_W8)
+
+
+@pytest.mark.parametrize("kernel_variant", [16, 32], indirect=True)
+def test_headline_shape_on_both_forms_of_the_256_row_kernel(kernel_variant):
+    # the whole headline shape forced onto each form (8 of its 32 slices against the oracle; the default form is checked on
+    # all of them above)
+    B, H, S, D = 2, 16, 8192, 128
+    q, k, v = _qkv(B, H, S, S, D, torch.bfloat16, seed=0)
+    o, lse = multi_head_attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=True, return_lse=True)
+    torch.cuda.synchronize()
+    o, lse = o.cpu(), lse.cpu()
+    for b, h in [(0, 0), (0, 5), (0, 10), (0, 15), (1, 3), (1, 6), (1, 9), (1, 12)]:
+        o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], causal=True)
+        _check(o[b:b + 1, h:h + 1], lse[b:b + 1, h:h + 1], o_ref, lse_ref, f"variant {kernel_variant} slice ({b},{h})")
 
 
 @pytest.mark.parametrize("shape", [(1, 8, 1300, 1300), (2, 8, 800, 1000), (3, 8, 1111, 900), (1, 16, 1537, 1537)])
