@@ -8,7 +8,7 @@
 // fp32 scores and accumulators; P and dS are rounded to the operand type before the second GEMMs, as the reference
 // does (:515,:562-563).
 //
-// Two launches, no atomics, no scratch beyond the caller's [B, H, Sq] fp32 `delta` buffer:
+// Two launches, no atomics, no scratch beyond the caller's [2, B, H, Sq] fp32 workspace (delta and -LSE / scale):
 //   1. attn_bwd_dq_kernel: one workgroup per 128 query rows (4 waves x 32), walks the key tiles like the forward
 //      kernel. Scores are computed transposed, S^T = K Q^T and dP^T = V dO^T (A operands = K / V rows from LDS, B
 //      operands = Q^T / dO^T held in registers), so a lane owns one query: LSE and delta are per-lane scalars and
@@ -41,11 +41,12 @@ struct AttnBwdParams {
   const void *q, *k, *v, *o, *d_o;
   const float* lse;
   float* delta;
+  float* nlse;        // [B, H, Sq]: -LSE / softmax_scale, written by the dQ kernel beside delta (see there)
   void *dq, *dk, *dv;
   int B, H, Sq, Sk;
   int d;                // true head_dim: a multiple of 8, at most the D the kernels are compiled for
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];   // element strides: batch, head, sequence
-  float scale, scale_log2e;
+  float scale, scale_log2e, neg_inv_scale_log2e;   // softmax scale, scale * log2 e, -1 / (scale * log2 e)
   int head_group;       // heads per group in the order of the workgroups (see bwd_item)
   DropoutParams drop;   // used by the kernels instantiated with dropout only
   BiasParams bias;      // used by the kernels instantiated with bias only
@@ -74,6 +75,15 @@ constexpr float kLog2e = 1.4426950408889634f;
 // falls back to FO_MFMA_NOPS=1, the builtin, if it finds a violation.
 #ifndef FO_MFMA_NOPS
 #define FO_MFMA_NOPS 0
+#endif
+// pipelined dK/dV kernel: the copies of the tile after next are issued between the MFMAs of phase 4 (1) or in one batch
+// at the hand-over (0)
+#ifndef FO_BWD_SPREAD
+#define FO_BWD_SPREAD 1
+#endif
+// ... its score accumulators start from -LSE / scale: never (0), at head_dim <= 64 (1), always (2)
+#ifndef FO_BWD_NLSE
+#define FO_BWD_NLSE 1
 #endif
 template <typename T>
 __device__ __forceinline__ void mfma_acc_agpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b) {
@@ -432,6 +442,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   // stores take, and staging the rows in LDS as the dK/dV kernels do made this kernel 5-10 % slower)
   const int qi = q0w + l32;
   if (qi < Sq) {
+    // -LSE / softmax_scale for the dK/dV kernel, whose score accumulators start from it: P = exp2((QK^T - LSE / scale)
+    // * scale * log2 e) is then one multiplication and the exponential per element. (Stored here, from the scaled LSE
+    // the loop used, and not beside delta: every register is taken while the loop runs.)
+    if (hh == 0) prm.nlse[(int64_t)bh * Sq + qi] = lse2 * prm.neg_inv_scale_log2e;
     T* op = (T*)prm.dq + b * prm.dqs[0] + h * prm.dqs[1] + (int64_t)qi * prm.dqs[2];
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
@@ -692,6 +706,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   static_assert(4 * DBLK == NMF && EPG >= 1, "phases of equal length");
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   constexpr int NBUF = 3;                   // tile buffers: see hand_over()
+  // the score accumulators start from -LSE / scale (see start_dp) instead of LSE being subtracted per element: one
+  // VALU instruction per element less. Measured at the socket power limit, on random operands: head_dim 64 -2 % time;
+  // head_dim 128 -4 % cycles and +4 % time (the chip clocks that form 10 % lower), so there it is left off.
+  constexpr bool NLSE = FO_BWD_NLSE == 2 || (FO_BWD_NLSE == 1 && D <= 64);
   FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q[NBUF] | dO[NBUF] | lse[NBUF][64] | delta[NBUF][64]
   FO_LDS float* rowvals = (FO_LDS float*)(smem + 2 * NBUF * TILE_BYTES);
   const int tid = threadIdx.x;
@@ -709,6 +727,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;     // queries before the block's first key never attend it
   const int ja = CAUSAL ? min(k0w / kBwdTile, n_qt) : 0;     // ... and this wave's keys start later still
 
+  const float* lse_src = NLSE ? (const float*)prm.nlse : prm.lse;
   TileLaneOffsets<T, D> qlo, glo;
   qlo.init(prm.qs[2], prm.d, wave_s, lane);
   glo.init(prm.dos[2], prm.d, wave_s, lane);
@@ -722,7 +741,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     }
     if (wave_s < 2) {
       const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
-      dma4_lane_ptr((wave_s == 0 ? prm.lse : (const float*)prm.delta) + at, rowvals + (NBUF * wave_s + buf) * kBwdTile);
+      dma4_lane_ptr((wave_s == 0 ? lse_src : (const float*)prm.delta) + at, rowvals + (NBUF * wave_s + buf) * kBwdTile);
     }
   };
   if (qt0 < n_qt) issue(qt0, 0);
@@ -808,8 +827,14 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   i32x4 pf[2][2], dsf[2][2];
   float p_even[2] = {0.0f, 0.0f}, ds_even[2] = {0.0f, 0.0f};
 
-  auto tile_body = [&](int j, auto masked) {
-    const int buf = (j - qt0) % NBUF, nbuf = (buf + 1) % NBUF;
+  const uint32_t lane4 = (uint32_t)lane * 4u;
+  // `buf`: the tile's buffer, (j - qt0) % NBUF, which the caller counts along.
+  // `spread`: tile j+2 lies wholly inside Q and dO (and the lane offsets fit): its copy is not issued in one batch at
+  // the hand-over but one instruction at a time between the MFMAs of phase 4 (a batch of direct-to-LDS copies holds the
+  // wave's issue port for hundreds of cycles while the matrix pipe runs dry; one copy per two MFMAs hides behind them)
+  auto tile_body = [&](int j, int buf, auto masked, auto spread) {
+    constexpr bool SPREAD = decltype(spread)::value;
+    const int nbuf = buf == NBUF - 1 ? 0 : buf + 1;
     const int q0t = j * kBwdTile;
     uint32_t rq[KSTEPS], cq[DBLK][2], rq_next[(kFragAhead + 1) / 2];
 #pragma unroll
@@ -834,7 +859,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     f32x4 lv[2];               // LSE of four query rows, fetched one vector ahead
     // dP = dO V^T - delta comes out of the MFMAs: the accumulator of a block's dP starts from -delta of its 16 rows,
     // read from LDS straight into the accumulator registers while they are idle (block 1: during phase 1; block 0 of
-    // the next tile: during phase 4, after the hand-over made that tile visible)
+    // the next tile: during phase 4, after the hand-over made that tile visible). The block's scores start from
+    // -LSE / scale in the same way, so that QK^T - LSE / scale comes out of the MFMAs.
     auto start_dp = [&](f32x16& acc, FO_LDS const float* del, int qb) {
 #pragma unroll
       for (int jv = 0; jv < 4; ++jv) {
@@ -847,7 +873,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     // dead iff key > query or the query is past the end
     auto element = [&](int qb, int r) {
       const int jv = r >> 2, u = r & 3;
-      if (u == 0 && jv + 1 < 4) {
+      if (!NLSE && u == 0 && jv + 1 < 4) {
         lv[(jv + 1) & 1] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * (jv + 1) + 4 * hh);
       }
       const int koff = u + 8 * jv;
@@ -857,7 +883,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
         const int lim_end = Sq - (q0t + 32 * qb + 4 * hh);
         dead = koff < lim || koff >= lim_end;
       }
-      const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][r], c, -lv[jv & 1][u] * kLog2e));
+      // (with NLSE the score accumulator started from -LSE / scale: see start_dp)
+      const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(NLSE ? sacc[qb][r] * c : __builtin_fmaf(sacc[qb][r], c, -lv[jv & 1][u] * kLog2e));
       const float ds = p * dpacc[qb][r];   // (dP - delta) softmax_scale is applied to the finished dK
       if (r & 1) {
         // a finished pair is rounded and pinned to its micro-group: left alone, the compiler moves the multiplication
@@ -874,16 +901,17 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       }
     };
     auto first_rows = [&](int qb) {
-      lv[0] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 4 * hh);
+      if (!NLSE) lv[0] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 4 * hh);
     };
     // ---- phase 1
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = i;
-      if (i & 1) mfma_scores_vgpr<T>(dpacc[0], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[0], fr[g % kFragAhead], kf[i >> 1], i == 0);
+      if (i & 1) mfma_scores_vgpr<T>(dpacc[0], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[0], fr[g % kFragAhead], kf[i >> 1], i == 0 && !NLSE);
       refill(g);
       if (i == 0) start_dp(dpacc[1], del_t, 1);
+      if (NLSE && i == 1) start_dp(sacc[1], lse_t, 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- phase 2
@@ -891,7 +919,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 #pragma unroll
     for (int i = 0; i < NMF; ++i) {
       const int g = NMF + i;
-      if (i & 1) mfma_scores_vgpr<T>(dpacc[1], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[1], fr[g % kFragAhead], kf[i >> 1], i == 0);
+      if (i & 1) mfma_scores_vgpr<T>(dpacc[1], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[1], fr[g % kFragAhead], kf[i >> 1], i == 0 && !NLSE);
       refill(g);
       if (i == 0) scores_fence(sacc[0], dpacc[0]);
 #pragma unroll
@@ -911,7 +939,23 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       for (int e = 0; e < EPG; ++e) element(1, i * EPG + e);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (j + 1 < n_qt) hand_over(j);
+    const char* next_q = nullptr;
+    const char* next_g = nullptr;
+    const char* next_rows = nullptr;
+    uint32_t next_q_dst = 0;
+    FO_LDS char* next_rows_dst = nullptr;
+    if constexpr (SPREAD) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      const int b2 = buf == 0 ? NBUF - 1 : buf - 1, which = wave_s & 1;   // (waves 2 and 3 repeat the row values of waves 0 and 1)
+      next_q = (const char*)(qbase + (int64_t)(j + 2) * kBwdTile * prm.qs[2]);
+      next_g = (const char*)(gbase + (int64_t)(j + 2) * kBwdTile * prm.dos[2]);
+      next_rows = (const char*)((which ? (const float*)prm.delta : lse_src) + (int64_t)bh * Sq + (j + 2) * kBwdTile);
+      next_q_dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem + b2 * TILE_BYTES + wave_s * (TileLaneOffsets<T, D>::N * 1024)));
+      next_rows_dst = (FO_LDS char*)(rowvals + (NBUF * which + b2) * kBwdTile);
+    } else {
+      if (j + 1 < n_qt) hand_over(j);
+    }
     // ---- phase 4
     // (two wait states: the paths around the hand-over join here, and the check of the generated code, which follows
     // no branches, must see that the first MFMA does not read a register written by the VALU instruction before it)
@@ -923,6 +967,29 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, dsf[1][t])); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, pf[1][t]));
       refill(g);
       if (i == 0) start_dp(dpacc[0], rowvals + (NBUF + nbuf) * kBwdTile, 0);   // (after the last tile: read, unused)
+      if (NLSE && i == 1) start_dp(sacc[0], rowvals + nbuf * kBwdTile, 0);
+      if constexpr (SPREAD) {
+        constexpr int N = TileLaneOffsets<T, D>::N, EVERY = NMF / (2 * N);
+        static_assert(EVERY >= 1 && 2 * N * EVERY == NMF && 2 * N <= 8, "one copy per EVERY micro-groups");
+        auto copy_piece = [&](auto pc) {
+          constexpr int piece = decltype(pc)::value;
+          if constexpr (piece < N) dma16_uniform_base_lds_imm<piece * 1024>(next_q, qlo.off[piece], next_q_dst);
+          else if constexpr (piece < 2 * N) dma16_uniform_base_lds_imm<NBUF * TILE_BYTES + (piece - N) * 1024>(next_g, glo.off[piece - N], next_q_dst);
+        };
+        if (i % EVERY == EVERY - 1) {
+          switch (i / EVERY) {      // (a constant once the loop is unrolled)
+            case 0: copy_piece(std::integral_constant<int, 0>{}); break;
+            case 1: copy_piece(std::integral_constant<int, 1>{}); break;
+            case 2: copy_piece(std::integral_constant<int, 2>{}); break;
+            case 3: copy_piece(std::integral_constant<int, 3>{}); break;
+            case 4: copy_piece(std::integral_constant<int, 4>{}); break;
+            case 5: copy_piece(std::integral_constant<int, 5>{}); break;
+            case 6: copy_piece(std::integral_constant<int, 6>{}); break;
+            default: copy_piece(std::integral_constant<int, 7>{}); break;
+          }
+        }
+        if (i == 0) dma4_uniform_base(next_rows, lane4, next_rows_dst);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -947,11 +1014,23 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       const f32x4 d4 = *(FO_LDS const f32x4*)(rowvals + (NBUF + buf) * kBwdTile + 8 * jv + 4 * hh);
 #pragma unroll
       for (int u = 0; u < 4; ++u) dpacc[0][4 * jv + u] = d4[u];
+      if constexpr (NLSE) {
+        const f32x4 n4 = *(FO_LDS const f32x4*)(rowvals + buf * kBwdTile + 8 * jv + 4 * hh);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sacc[0][4 * jv + u] = n4[u];
+      }
     }
   }
-  for (; j < n_qt && needs_mask(j); ++j) tile_body(j, std::true_type{});
-  for (; j < n_qt && !needs_mask(j); ++j) tile_body(j, std::false_type{});
-  for (; j < n_qt; ++j) tile_body(j, std::true_type{});
+  int buf = j < n_qt ? (j - qt0) % NBUF : 0;
+  auto next_buf = [&]() { buf = buf == NBUF - 1 ? 0 : buf + 1; };
+  for (; j < n_qt && needs_mask(j); ++j, next_buf()) tile_body(j, buf, std::true_type{}, std::false_type{});
+#if FO_BWD_SPREAD
+  // (from here on only a last tile that crosses the end of Q needs the mask; tiles j with tile j+2 wholly inside Q)
+  if (qlo.ok && glo.ok)
+    for (const int end = Sq / kBwdTile - 2; j < end; ++j, next_buf()) tile_body(j, buf, std::false_type{}, std::true_type{});
+#endif
+  for (; j < n_qt && !needs_mask(j); ++j, next_buf()) tile_body(j, buf, std::false_type{}, std::false_type{});
+  for (; j < n_qt; ++j, next_buf()) tile_body(j, buf, std::true_type{}, std::false_type{});
 
   acc_fence(dkacc);
   acc_fence(dvacc);
@@ -1008,11 +1087,11 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
 
 using namespace fo;
 
-// ---- the same without a workspace argument and without any allocation: delta lives in a device array of this library.
+// ---- the same without a workspace argument and without any allocation: the workspace is a device array of this library.
 // The array's name is only a host-side handle for the device symbol; its address on a device comes from
 // hipGetSymbolAddress, asked once per device with that device current, and only that pointer is handed to the kernels.
 constexpr int64_t kStaticDeltaFloats = FO_ATTN_BWD_STATIC_ROWS;
-static __device__ __align__(256) float scratch[kStaticDeltaFloats];
+static __device__ __align__(256) float scratch[2 * kStaticDeltaFloats];   // two values per row: see AttnBwdParams
 constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mutex;
 static float* g_scratch_ptr[kMaxDevices];   // per device; null until that device's first call
@@ -1069,13 +1148,14 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
   }
 
   AttnBwdParams p;
-  p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse; p.delta = delta_ws; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.q = q; p.k = k; p.v = v; p.o = o; p.d_o = d_o; p.lse = lse; p.delta = delta_ws; p.nlse = delta_ws + (int64_t)B * H * Sq; p.dq = dq; p.dk = dk; p.dv = dv;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.d = D;
   int64_t* dst[8] = {p.qs, p.ks, p.vs, p.os, p.dos, p.dqs, p.dks, p.dvs};
   for (int t = 0; t < 8; ++t)
     for (int i = 0; i < 3; ++i) dst[t][i] = strides_host[t][i];
   p.scale = softmax_scale;
   p.scale_log2e = softmax_scale * kLog2e;
+  p.neg_inv_scale_log2e = -1.0f / p.scale_log2e;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool c = causal != 0, drop = dropout_p > 0.0f;
   p.drop = make_dropout(dropout_p, seed, rng_offset);

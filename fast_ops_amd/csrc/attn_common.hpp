@@ -42,6 +42,13 @@ __device__ __forceinline__ void dma16_uniform_base(const void* base, uint32_t by
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(byte_off), "s"(base) : "memory", "m0");
 #endif
 }
+// ... with the LDS address as a wave-uniform register plus a constant: one scalar instruction forms it in M0
+template <int IMM>
+__device__ __forceinline__ void dma16_uniform_base_lds_imm(const void* base, uint32_t byte_off, uint32_t lds_base) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(byte_off), "s"(base), "n"(IMM) : "memory", "m0", "scc");
+#endif
+}
 __device__ __forceinline__ void dma16_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
@@ -112,6 +119,12 @@ __device__ __forceinline__ void load_bias4(const E* at, float* out) {
 __device__ __forceinline__ void dma4_lane_ptr(const void* ptr, FO_LDS void* dst) {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(ptr) : "memory", "m0");
+#endif
+}
+// ... from a wave-uniform base plus a per-lane byte offset
+__device__ __forceinline__ void dma4_uniform_base(const void* base, uint32_t byte_off, FO_LDS void* dst) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst)), "v"(byte_off), "s"(base) : "memory", "m0");
 #endif
 }
 

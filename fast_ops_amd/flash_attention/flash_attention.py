@@ -215,7 +215,7 @@ def attn_bwd_strided(
     dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-    delta = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    delta = torch.empty((2, B, H, Sq), dtype=torch.float32, device=q.device)   # workspace: -delta and -LSE / scale per row
     if bias is not None:
         bias = _expand_bias(bias, q, B, H, Sq, Sk)
     tensors = (q, k, v, o, d_o, dq, dk, dv)

@@ -107,7 +107,8 @@ int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* k_str
  *
  *   q, k, v, o, lse     as passed to / produced by fo_attn_fwd (lse is required here)
  *   d_o                 [B, H, Sq, D] gradient of the output
- *   delta_ws            [B, H, Sq] fp32, contiguous: workspace supplied by the caller, overwritten
+ *   delta_ws            [2, B, H, Sq] fp32, contiguous: workspace supplied by the caller, overwritten (per query row
+ *                       -delta and -LSE / scale, written by the first launch for the second)
  *   dq / dk, dv         [B, H, Sq, D] / [B, H, Sk, D], written for every element; never read
  *   strides_host        eight pointers to three element strides each (batch, head, sequence; head_dim stride 1), in
  *                       the order q, k, v, o, d_o, dq, dk, dv. Only the inputs may repeat a batch or head (stride 0).
@@ -120,8 +121,8 @@ int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, cons
 
 /* fo_attn_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): no workspace argument, and the call itself allocates and frees nothing. The
- * [B, H, Sq] fp32 delta buffer lives in a device array of the library (FO_ATTN_BWD_STATIC_ROWS floats = 4 MiB, which
- * each GPU the library runs on holds until the process ends). B*H*Sq above FO_ATTN_BWD_STATIC_ROWS is refused with
+ * [2, B, H, Sq] fp32 workspace lives in a device array of the library (2 * FO_ATTN_BWD_STATIC_ROWS floats = 8 MiB,
+ * which each GPU the library runs on holds until the process ends). B*H*Sq above FO_ATTN_BWD_STATIC_ROWS is refused with
  * FO_ERR_BAD_SHAPE. Same results as fo_attn_bwd, bit for bit. All calls on one GPU share the array: calls that
  * overlap on one GPU (different streams or threads) race on it and must be serialised by the caller; calls in stream
  * order on one stream are safe. The first call on a device looks up the array's address there (hipGetSymbolAddress;

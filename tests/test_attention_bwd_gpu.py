@@ -222,7 +222,7 @@ def test_columns_past_the_head_dim_are_neither_read_nor_written(D, row, causal):
     rc = _lib.load().fo_attn_fwd(qw.data_ptr(), kw.data_ptr(), vw.data_ptr(), o_out.data_ptr(), lse2.data_ptr(), B, H, Sq, Sk, D,
                                  st(qw), st(kw), st(vw), st(o_out), sc, int(causal), _lib.FO_DTYPE_BF16, stream)
     assert rc == 0, _lib.strerror(rc)
-    delta = torch.empty(B, H, Sq, dtype=torch.float32, device=DEV)
+    delta = torch.empty(2, B, H, Sq, dtype=torch.float32, device=DEV)
     tensors = (qw, kw, vw, ow, gw, outs[0], outs[1], outs[2])
     arrays = [st(t) for t in tensors]
     strides = (P64 * 8)(*[ctypes.cast(a, P64) for a in arrays])

@@ -56,7 +56,7 @@ CALLS = [
 def test_static_workspace_backward_equals_the_workspace_argument_form(calls):
     for i, (B, H, Sq, Sk, D, dtype, causal) in enumerate(calls):
         q, k, v, o, lse, go = _inputs(B, H, Sq, Sk, D, dtype, causal, seed=17 + i)
-        delta = torch.empty(B, H, Sq, dtype=torch.float32, device=DEV)
+        delta = torch.empty(2, B, H, Sq, dtype=torch.float32, device=DEV)
         want = _backward("fo_attn_bwd", q, k, v, o, lse, go, causal, delta)
         torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
