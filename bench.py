@@ -370,6 +370,91 @@ def bench_clock(steps, warmup, settle):
     return out
 
 
+def bench_power(seconds):
+    """Socket power while each kernel runs back to back for `seconds`: the attention forward of the headline shape on
+    standard-normal and on all-zero operands, its backward, the vendor library's GEMM on both kinds of operands, and the
+    fused Lion step. Power is the amdgpu driver's own sensor (hwmon power1_input or power1_average of the card, in
+    microwatts), read every 10 ms by a host thread; a kernel's figure is the mean over its loop without the first second.
+    Beside it the time per launch over the same loop, by events."""
+    import glob
+    import threading
+
+    import torch
+
+    from fast_ops.flash_attention.flash_attention import multi_head_attention
+    from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided, attn_fwd_strided
+
+    sensors = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")) or \
+        sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
+    if not sensors:
+        print("bench.py --path power: no power sensor under /sys/class/drm/card*/device/hwmon", file=sys.stderr)
+        sys.exit(2)
+    sensor = sensors[0]
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                samples.append((time.perf_counter(), int(open(sensor).read()) * 1e-6))
+            except (OSError, ValueError):
+                pass
+            time.sleep(0.01)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    dev, B, H, S, D = "cuda:0", 2, 16, 8192, 128
+    scale = 1.0 / (D ** 0.5)
+    (q, k, v), g = _attn_inputs(B, H, S, D, torch.bfloat16, dev)
+    go = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(dev)
+    o, lse = attn_fwd_strided(q, k, v, (0, 1, 2, 3), True, scale)
+    zq = torch.zeros_like(q)
+    n = 8192
+    a, b = (torch.randn(n, n, generator=g).to(torch.bfloat16).to(dev) for _ in range(2))
+    za = torch.zeros_like(a)
+    _params, opt = _lion_setup(LION_LARGE_SHAPES, dev)
+    cases = [
+        ("attention forward, standard-normal operands", lambda: multi_head_attention(q, k, v, causal=True, softmax_scale=scale), 2.0 * B * H * S * S * D),
+        ("attention forward, all-zero operands", lambda: multi_head_attention(zq, zq, zq, causal=True, softmax_scale=scale), 2.0 * B * H * S * S * D),
+        ("attention backward, standard-normal operands", lambda: attn_bwd_strided(q, k, v, o, lse, go, (0, 1, 2, 3), True, scale), 5.0 * B * H * S * S * D),
+        ("library GEMM 8192^3 bf16, standard-normal operands", lambda: torch.matmul(a, b), 2.0 * n ** 3),
+        ("library GEMM 8192^3 bf16, all-zero operands", lambda: torch.matmul(za, za), 2.0 * n ** 3),
+        ("fused Lion step, 1.3 B parameters", lambda: opt.step(), None),
+    ]
+    torch.cuda.synchronize()
+    time.sleep(1.0)
+    t_idle_end = time.perf_counter()
+    out = {"sensor": sensor, "seconds_per_kernel": seconds, "kernels": []}
+    for name, step, flops in cases:
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = _events(2)
+        t0 = time.perf_counter()
+        launches = 0
+        e0.record()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                step()
+            launches += 20
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        watts = [w for t, w in samples if t0 + min(1.0, seconds / 2) <= t <= t1]
+        ms = e0.elapsed_time(e1) / launches
+        row = {"kernel": name, "launches": launches, "ms_per_launch": ms, "socket_watts_mean": sum(watts) / max(len(watts), 1),
+               "socket_watts_max": max(watts) if watts else None, "samples": len(watts)}
+        if flops is not None:
+            row["tflops"] = flops / (ms * 1e-3) / 1e12
+        out["kernels"].append(row)
+        time.sleep(0.5)
+    stop.set()
+    th.join()
+    idle = [w for t, w in samples if t <= t_idle_end]
+    out["socket_watts_idle"] = sum(idle) / max(len(idle), 1)
+    return out
+
+
 def bench_ablations(steps, warmup, settle):
     """Timing ablations of the 256-row attention kernel at the headline shape: what each part of the kernel costs in
     cycles and in clock. Needs a library built with `python -m fast_ops_amd.build --ablations` (the variants leave work
@@ -408,9 +493,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle", type=int, default=100,
                     help="clock-settle launches ahead of the warm-up of every timed section (reported, not counted as warm-up)")
-    ap.add_argument("--path", choices=["both", "attn", "lion", "copy", "clock", "ablations"], default="both",
+    ap.add_argument("--path", choices=["both", "attn", "lion", "copy", "clock", "power", "ablations"], default="both",
                     help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
                          "clock: the attention kernel against the number of busy CUs and the operand bits, with the library GEMM; "
+                         "power: socket power (the driver's sensor) while each kernel loops for 3 s; "
                          "ablations: the attention kernel with parts left out (needs a build with --ablations)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
@@ -438,6 +524,9 @@ def main():
         return
     if args.path == "clock":
         print(json.dumps(bench_clock(args.steps, args.warmup, args.settle)))
+        return
+    if args.path == "power":
+        print(json.dumps({"path": "power", **bench_power(3.0)}))
         return
     if args.path == "ablations":
         print(json.dumps(bench_ablations(args.steps, args.warmup, args.settle)))
