@@ -1142,17 +1142,27 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
   // 128-row kernel, with four times as many workgroups, fills the chip better
   static const int n_cu = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256; return n; }();
   const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
-  // (causal, up to 2048 queries: a 256-row block is a large part of the triangle, and the 128-row kernel with its finer
-  // blocks, heaviest first, is 10-20 % faster at 1024 queries and equal or a few per cent faster at 2048)
   int v = forced;
   if (forced < 0) {
-    v = (wide_ok && wide_wgs >= n_cu && !(causal && p.Sq <= 2048)) ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128;
+    const int keys = causal ? (p.Sq < p.Sk ? p.Sq : p.Sk) : p.Sk;
+    // One workgroup per CU at a time: the launch runs in rounds, and a last round that is mostly empty is paid in full.
+    // With the rounds filled to less than 80 % the 128-row kernel (two workgroups per CU, finer blocks, heaviest first)
+    // was 1-5 % faster (B*H = 160-192 at 512-1024 keys, 48 heads x 4096 causal), from 83 % on the 256-row kernel 3-6 %.
+    const int64_t rounds = (wide_wgs + n_cu - 1) / n_cu;
+    bool wide = wide_ok && wide_wgs >= n_cu && wide_wgs * 5 >= rounds * n_cu * 4;
+    // head_dim 128, causal: from 1024 queries on (B*H = 128: 1024 queries -8 %, 1536 -16 %, 2048 -12 % against the
+    // 128-row kernel; 512 and 768 queries +7 % and +18 %, a 256-row block being a large part of so small a triangle).
+    if (D == 128 && causal && p.Sq < 1024) wide = false;
+    // head_dim 64 (half the MFMAs per score, so the softmax weighs twice as much and the 128-row kernel's two workgroups
+    // per CU hide it better): only for long rows of keys. Non-causal 1024 keys +20 %, 2048 +5 %, 4096 +0.6 %, 8192
+    // -0.5 %, 16384 -1.8 %; causal 2048 +10 %, 4096 +6.6 %, 6144 +5.5 %, 8192 +1.5 %, 16384 -1.2 %.
+    if (D == 64 && keys < (causal ? 16384 : 8192)) wide = false;
+    v = wide ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128;
     // head_dim 128 with many key tiles per query block: four waves x 64 rows. Every K / V^T fragment read from LDS feeds two
     // MFMAs, which costs less energy (at full load the chip's clock is what its power budget leaves) but more cycles per
     // tile, and its longer pipeline fill and drain have to be spread over enough tiles. Measured on one box, new form
     // against the eight-wave form: non-causal 2048 keys -1.0 %, 4096 -2.3 %, 8192 -2.5 %; causal 3072 +3 %, 4096 +1 %,
     // 8192 -0.7 %, 16384 -1.8 %.
-    const int keys = causal ? (p.Sq < p.Sk ? p.Sq : p.Sk) : p.Sk;
     if (v == FO_ATTN_KERNEL_ROWS256_W8 && D == 128 && keys >= (causal ? 6144 : 2048)) v = FO_ATTN_KERNEL_ROWS256_W4;
   }
   if (v >= 256) return v;

@@ -217,13 +217,38 @@ def test_ragged_across_256_row_blocks_head_dim_64(shape, causal, dtype, kernel_v
     _run_and_check(B, H, Sq, Sk, 64, dtype, causal, seed=Sq + Sk + 64)
 
 
-@pytest.mark.parametrize("causal,S", [(True, 2304), (False, 1024)])
-def test_head_dim_64_large_shape_takes_the_256_row_kernel_by_default(causal, S):
-    # enough 256-row workgroups for every CU (80 heads x 5 pairs of query blocks, the middle one single / x 4 blocks), and
-    # more than 2048 queries where causal: the library's own choice is the 256-row kernel, and must agree with the oracle
-    q, k, v = _qkv(2, 40, S, S, 64, torch.bfloat16, seed=5)
+@pytest.mark.parametrize("causal,S", [(True, 16384), (False, 8192)])
+def test_head_dim_64_long_shape_takes_the_256_row_kernel_by_default(causal, S):
+    # head_dim 64 takes the 256-row kernel only for long rows of keys (8192 non-causal, 16384 causal) and one workgroup
+    # per CU (8 heads x 32 blocks / pairs of blocks): the library's own choice, and it must agree with the oracle
+    q, k, v = _qkv(1, 8, S, S, 64, torch.bfloat16, seed=5)
     assert _kernel_taken(q, k, v, causal) == _lib.FO_ATTN_KERNEL_ROWS256_W8
+    _run_and_check(1, 8, S, S, 64, torch.bfloat16, causal, seed=5)
+
+
+@pytest.mark.parametrize("causal,S", [(True, 2304), (False, 1024)])
+def test_head_dim_64_shorter_shape_takes_the_128_row_kernel_by_default(causal, S):
+    q, k, v = _qkv(2, 40, S, S, 64, torch.bfloat16, seed=5)
+    assert _kernel_taken(q, k, v, causal) == _lib.FO_ATTN_KERNEL_ROWS128
     _run_and_check(2, 40, S, S, 64, torch.bfloat16, causal, seed=5)
+
+
+@pytest.mark.parametrize("heads,expect", [(128, "rows256_w8"), (192, "rows128")])
+def test_short_causal_head_dim_128_choice_follows_the_fill_of_the_rounds(heads, expect):
+    # B*H heads x 1024 queries, causal: two workgroups of two 256-row blocks per head. 128 heads fill the 256 CUs once
+    # (256-row kernel); 192 heads would leave half of a second round empty (128-row kernel). Checked against the oracle
+    # on a sample of heads that covers every XCD.
+    B, H, S, D = heads // 16, 16, 1024, 128
+    q, k, v = _qkv(B, H, S, S, D, torch.bfloat16, seed=heads)
+    want = {"rows256_w8": _lib.FO_ATTN_KERNEL_ROWS256_W8, "rows128": _lib.FO_ATTN_KERNEL_ROWS128}[expect]
+    assert _kernel_taken(q, k, v, True) == want
+    o, lse = multi_head_attention(q.to(DEV), k.to(DEV), v.to(DEV), causal=True, return_lse=True)
+    torch.cuda.synchronize()
+    o, lse = o.cpu(), lse.cpu()
+    for i in range(0, heads, 11):
+        b, h = divmod(i, H)
+        o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], causal=True)
+        _check(o[b:b + 1, h:h + 1], lse[b:b + 1, h:h + 1], o_ref, lse_ref, f"{expect} head {i}")
 
 
 def test_causal_up_to_2048_queries_takes_the_128_row_kernel_by_default():

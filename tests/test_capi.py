@@ -191,6 +191,18 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     finally:
         lib.fo_tune_set(b"attn.variant", -1)
     assert k(1, 1, 128, 128, 76, 0) == -3 and k(0, 1, 128, 128, 64, 0) == -4
+    # the library's own choice on 256 CUs (an MI355X, or what the library assumes where it finds no device)
+    R128, W8, W4 = _lib.FO_ATTN_KERNEL_ROWS128, _lib.FO_ATTN_KERNEL_ROWS256_W8, _lib.FO_ATTN_KERNEL_ROWS256_W4
+    assert k(2, 16, 8192, 8192, 128, 1) == W4            # the headline shape: 512 workgroups of two query blocks
+    assert k(16, 32, 2048, 2048, 128, 0) == W4           # B=16 H=32 S=2048 non-causal
+    assert k(8, 12, 1024, 1024, 64, 1) == R128           # the GPT-2-small shape
+    assert k(2, 16, 4096, 4096, 128, 1) == W8            # fewer than 6144 keys, causal: eight waves
+    assert k(8, 16, 1024, 1024, 128, 1) == W8            # causal from 1024 queries on: 256 workgroups, one round
+    assert k(12, 16, 1024, 1024, 128, 1) == R128         # 384 workgroups would leave half of the second round empty
+    assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
+    assert k(16, 16, 512, 512, 128, 0) == W8 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups
+    assert k(1, 8, 8192, 8192, 64, 0) == W8 and k(2, 8, 4096, 4096, 64, 0) == R128     # head_dim 64: long rows only
+    assert k(1, 8, 16384, 16384, 64, 1) == W8 and k(1, 16, 8192, 8192, 64, 1) == R128
     # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
     assert k(2, 16, 8192, 8192, 96, 1) == _lib.FO_ATTN_KERNEL_ROWS128
     assert lib.fo_attn_fwd_kernel(1, 1, 128, 128, 64, None, dense(128, 64), 0, 0, 0) == -1
