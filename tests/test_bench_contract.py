@@ -1,5 +1,5 @@
 """bench.py's contract with its caller: one JSON line on stdout with the agreed keys, one GPU only, and the workload
-constants it is quoted on (BASELINE.json: attention forward B=2 H=16 S=8192 D=128 bf16 causal; Lion over 1.3 B
+constants it is quoted on (attention forward B=2 H=16 S=8192 D=128 bf16 causal; Lion over 1.3 B
 parameters; the GPT-2-small sets of the reference's own benchmarks, benchmarks/benchmark_lion.py:10-16 and
 benchmarks/benchmark_flash_attention.py:195-209)."""
 import json
