@@ -111,6 +111,25 @@ def test_long_context_slice_of_headline_shape(causal, dkdv_variant):
         assert math.isfinite(e) and e <= 2e-2 * max(1.0, r.abs().max().item()), f"{name}: error {e:.3e} vs magnitude {r.abs().max().item():.3e}"
 
 
+def test_headline_shape_whole_with_the_benchmarks_dispatch():
+    # B=2 H=16 S=8192 D=128 bf16 causal as bench.py runs it: 32 heads dealt to the 8 XCDs, 64 key blocks and 64 query
+    # blocks per head, the library's own choice of kernels and workgroup order. Six (batch, head) slices that lie on six
+    # different XCDs, first and last head included, against the fp32 closed form (absolute criterion as above).
+    B, H, S, D = 2, 16, 8192, 128
+    q, k, v, go = _inputs(B, H, S, S, D, torch.bfloat16, seed=4)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    o = multi_head_attention(qd, kd, vd, causal=True)
+    got = [g.cpu() for g in torch.autograd.grad(o, (qd, kd, vd), go.to(DEV))]
+    slices = [(0, 0), (0, 5), (0, 10), (1, 3), (1, 9), (1, 15)]
+    assert len({(b * H + h) % 8 for b, h in slices}) == 6
+    for b, h in slices:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = attention_bwd_oracle(q[sl], k[sl], v[sl], go[sl], causal=True)
+        for name, a, r in zip(("dQ", "dK", "dV"), got, ref):
+            e = (a[sl].float() - r).abs().max().item()
+            assert math.isfinite(e) and e <= 2e-2 * max(1.0, r.abs().max().item()), f"slice ({b},{h}) {name}: error {e:.3e} vs magnitude {r.abs().max().item():.3e}"
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 7, 5), (2, 1, 100, 100), (1, 3, 129, 257), (1, 2, 257, 129), (1, 1, 64, 300),
                                    (1, 1, 300, 64), (2, 2, 191, 191), (1, 1, 385, 513)])
 @pytest.mark.parametrize("causal", [False, True])
