@@ -64,19 +64,23 @@ def build_chunk_table(ptrs: List[Tuple[int, int, int, int]], p_size: int = 4, m_
     """(p_ptr, g_ptr, m_ptr, numel) per tensor -> structured array of fo_lion_chunk descriptors; p_size / m_size are
     the element sizes of parameters (and gradients) and of the momentum."""
     C = _lib.FO_LION_CHUNK
-    parts = []
-    for p_ptr, g_ptr, m_ptr, numel in ptrs:
-        if numel == 0:
-            continue
-        n = (numel + C - 1) // C
-        off = np.arange(n, dtype=np.uint64) * np.uint64(C)
-        t = np.zeros(n, dtype=_CHUNK_DTYPE)
-        t["p"] = np.uint64(p_ptr) + off * np.uint64(p_size)
-        t["g"] = np.uint64(g_ptr) + off * np.uint64(p_size)
-        t["m"] = np.uint64(m_ptr) + off * np.uint64(m_size)
-        t["n"] = np.minimum(np.uint64(C), np.uint64(numel) - off).astype(np.int32)
-        parts.append(t)
-    return np.concatenate(parts) if parts else np.zeros(0, dtype=_CHUNK_DTYPE)
+    # all tensors at once (a rebuild happens whenever a gradient comes back at another address, and a Python loop over
+    # the tensors took 3 ms for the 148 tensors of GPT-2-small)
+    arr = np.array([t for t in ptrs if t[3] != 0], dtype=np.uint64).reshape(-1, 4)
+    numel = arr[:, 3].astype(np.int64)
+    n = (numel + (C - 1)) // C                                  # chunks per tensor
+    total = int(n.sum())
+    t = np.zeros(total, dtype=_CHUNK_DTYPE)
+    if total == 0:
+        return t
+    first = np.cumsum(n) - n                                    # index of each tensor's first chunk
+    off = (np.arange(total, dtype=np.int64) - np.repeat(first, n)) * C      # element offset of the chunk in its tensor
+    off_u = off.astype(np.uint64)
+    t["p"] = np.repeat(arr[:, 0], n) + off_u * np.uint64(p_size)
+    t["g"] = np.repeat(arr[:, 1], n) + off_u * np.uint64(p_size)
+    t["m"] = np.repeat(arr[:, 2], n) + off_u * np.uint64(m_size)
+    t["n"] = np.minimum(C, np.repeat(numel, n) - off).astype(np.int32)
+    return t
 
 
 def lion_update(param: Tensor, grad: Tensor, exp_avg: Tensor, lr: float, beta1: float, beta2: float, weight_decay: float) -> None:
