@@ -39,10 +39,10 @@ SOURCES = {
     "capi.hip": [],
     "lion.hip": ["-ffp-contract=off"],
     "lion_typed.hip": ["-ffp-contract=off"],
-    # attn_fwd.hip lays its inner loop out as fully unrolled micro-groups; the default size limit for "#pragma unroll"
-    # would silently leave them rolled, with their register arrays in scratch memory.
+    # attn_fwd.hip and attn_bwd.hip lay their inner loops out as fully unrolled micro-groups; the default size limit for
+    # "#pragma unroll" would silently leave them rolled, with their register arrays in scratch memory.
     "attn_fwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
-    "attn_bwd.hip": [],
+    "attn_bwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
     "dropout_mask.hip": [],
 }
 # sources whose generated assembly is checked by asm_lint: source -> regular expression of the kernel symbols to check

@@ -81,10 +81,6 @@ constexpr float kLog2e = 1.4426950408889634f;
 #ifndef FO_BWD_SPREAD
 #define FO_BWD_SPREAD 1
 #endif
-// ... its score accumulators start from -LSE / scale: never (0), at head_dim <= 64 (1), always (2)
-#ifndef FO_BWD_NLSE
-#define FO_BWD_NLSE 1
-#endif
 template <typename T>
 __device__ __forceinline__ void mfma_acc_agpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b) {
 #if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
@@ -97,28 +93,15 @@ __device__ __forceinline__ void mfma_acc_agpr(f32x16& acc, typename Ops<T>::vec8
 #endif
 }
 // S / dP of the pipelined dK/dV kernel: result pinned in VGPRs (the softmax gradient reads it element by element; from
-// AGPRs every read is an extra instruction). `first` starts a new sum. Readers wait with scores_fence().
+// AGPRs every read is an extra instruction); the accumulator is given its start values before the first call. A VALU
+// instruction may read the result 11 wait states after the last MFMA was issued: the kernel's schedule sees to that.
 template <typename T>
-__device__ __forceinline__ void mfma_scores_vgpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b, bool first) {
+__device__ __forceinline__ void mfma_scores_vgpr(f32x16& acc, typename Ops<T>::vec8 a, typename Ops<T>::vec8 b) {
 #if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
-  if constexpr (std::is_same<T, __bf16>::value) {
-    if (first) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
-    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-  } else {
-    if (first) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
-    else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-  }
+  if constexpr (std::is_same<T, __bf16>::value) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 #else
-  if (first) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-  }
   acc = Ops<T>::mfma(a, b, acc);
-#endif
-}
-__device__ __forceinline__ void scores_fence(f32x16& s, f32x16& dp) {
-#if defined(__HIP_DEVICE_COMPILE__) && !FO_MFMA_NOPS
-  asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s), "+v"(dp));
 #endif
 }
 template <int N>
@@ -691,10 +674,12 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
 // two blocks of scores leave room for one wave per SIMD only, and a lone wave issues in order: whatever arithmetic sits
 // between two MFMAs keeps the matrix pipe waiting unless it is laid out to run beside them. A 64-query tile is two
 // 32-query blocks and four phases of NMF MFMAs each:
-//   1: S, dP of block 0 | 2: S, dP of block 1 + softmax gradient of block 0 | 3: dV, dK of block 0 + softmax gradient of
-//   block 1 | 4: dV, dK of block 1
-// as micro-groups of one MFMA, the LDS read of the A operand needed kFragAhead groups later and, in phases 2 and 3, one
-// or two score elements, fenced so that the compiler keeps the groups apart.
+//   1: S, then dP of block 0 | 2: S, then dP of block 1 | 3: dV, dK of block 0 | 4: dV, dK of block 1
+// as micro-groups of one MFMA, the LDS read of the A operand needed kFragAhead groups later and a share of the tile's
+// softmax-gradient arithmetic (see tile_body), fenced so that the compiler keeps the groups apart. The accumulators of
+// S and dP do not start from zero but from -LSE / scale and -delta of their rows (written by the dQ kernel, read from
+// LDS straight into the registers while they are idle), so that P = exp2((QK^T - LSE / scale) c) and dS = P (dP - delta)
+// are two multiplications and the exponential.
 template <typename T, int D, bool CAUSAL>
 __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
@@ -702,15 +687,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   constexpr int KSTEPS = D / 16;
   constexpr int DBLK = D / 32;
   constexpr int NMF = 2 * KSTEPS;           // MFMAs per phase (= 4 * DBLK)
-  constexpr int EPG = 16 / NMF;             // score elements per micro-group
-  static_assert(4 * DBLK == NMF && EPG >= 1, "phases of equal length");
+  static_assert(4 * DBLK == NMF, "phases of equal length");
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
   constexpr int NBUF = 3;                   // tile buffers: see hand_over()
-  // the score accumulators start from -LSE / scale (see start_dp) instead of LSE being subtracted per element: one
-  // VALU instruction per element less. Measured at the socket power limit, on random operands: head_dim 64 -2 % time;
-  // head_dim 128 -4 % cycles and +4 % time (the chip clocks that form 10 % lower), so there it is left off.
-  constexpr bool NLSE = FO_BWD_NLSE == 2 || (FO_BWD_NLSE == 1 && D <= 64);
-  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q[NBUF] | dO[NBUF] | lse[NBUF][64] | delta[NBUF][64]
+  FO_LDS char* smem = (FO_LDS char*)smem_raw;   // Q[NBUF] | dO[NBUF] | -LSE/scale[NBUF][64] | -delta[NBUF][64]
   FO_LDS float* rowvals = (FO_LDS float*)(smem + 2 * NBUF * TILE_BYTES);
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -727,7 +707,6 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   const int qt0 = CAUSAL ? min(k0 / kBwdTile, n_qt) : 0;     // queries before the block's first key never attend it
   const int ja = CAUSAL ? min(k0w / kBwdTile, n_qt) : 0;     // ... and this wave's keys start later still
 
-  const float* lse_src = NLSE ? (const float*)prm.nlse : prm.lse;
   TileLaneOffsets<T, D> qlo, glo;
   qlo.init(prm.qs[2], prm.d, wave_s, lane);
   glo.init(prm.dos[2], prm.d, wave_s, lane);
@@ -741,7 +720,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     }
     if (wave_s < 2) {
       const int64_t at = (int64_t)bh * Sq + min(qt * kBwdTile + lane, Sq - 1);
-      dma4_lane_ptr((wave_s == 0 ? lse_src : (const float*)prm.delta) + at, rowvals + (NBUF * wave_s + buf) * kBwdTile);
+      dma4_lane_ptr((wave_s == 0 ? (const float*)prm.nlse : (const float*)prm.delta) + at, rowvals + (NBUF * wave_s + buf) * kBwdTile);
     }
   };
   if (qt0 < n_qt) issue(qt0, 0);
@@ -805,10 +784,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       col_off[db][1] = (uint32_t)(r1 * ROW + ((chunk ^ swz<D>(r1)) * 16) + sub);
     }
   }
-  // A operand of MFMA i of a scores phase (even i: Q rows for S, odd i: dO rows for dP) / of a gradient phase (even i:
+  // A operand of MFMA i of a scores phase (i < KSTEPS: Q rows for S, then dO rows for dP) / of a gradient phase (even i:
   // dO^T for dV, odd i: Q^T for dK); rq / cq = the offsets above plus the byte offset of the tile's Q buffer
-  auto scores_frag = [&](const uint32_t* rq, int qb, int i) -> vec8 {
-    return *(FO_LDS const vec8*)(smem + rq[i >> 1] + ((i & 1) ? G_OFF : 0) + qb * 32 * ROW);
+  auto scores_frag_sd = [&](const uint32_t* rq, int qb, int i) -> vec8 {
+    return *(FO_LDS const vec8*)(smem + rq[i % KSTEPS] + (i >= KSTEPS ? G_OFF : 0) + qb * 32 * ROW);
   };
   auto grads_frag = [&](const uint32_t (*cq)[2], int qb, int i) -> vec8 {
     const int tp = 2 * qb + i / (2 * DBLK), db = (i >> 1) % DBLK;
@@ -825,18 +804,36 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   typedef __attribute__((ext_vector_type(4))) int i32x4;
   typedef __attribute__((ext_vector_type(2))) T vec2;
   i32x4 pf[2][2], dsf[2][2];
-  float p_even[2] = {0.0f, 0.0f}, ds_even[2] = {0.0f, 0.0f};
 
   const uint32_t lane4 = (uint32_t)lane * 4u;
-  // `buf`: the tile's buffer, (j - qt0) % NBUF, which the caller counts along.
-  // `spread`: tile j+2 lies wholly inside Q and dO (and the lane offsets fit): its copy is not issued in one batch at
-  // the hand-over but one instruction at a time between the MFMAs of phase 4 (a batch of direct-to-LDS copies holds the
-  // wave's issue port for hundreds of cycles while the matrix pipe runs dry; one copy per two MFMAs hides behind them)
-  auto tile_body = [&](int j, int buf, auto masked, auto spread) {
+  // One tile. `buf`: the tile's buffer, (j - qt0) % NBUF, which the caller counts along. `spread`: tile j+2 lies wholly
+  // inside Q and dO (and the lane offsets fit): its copy is not issued in one batch at the hand-over but one instruction
+  // at a time between the MFMAs of phase 4 (a batch of direct-to-LDS copies holds the wave's issue port for hundreds of
+  // cycles while the matrix pipe runs dry; one copy per two MFMAs hides behind them).
+  // The softmax-gradient arithmetic is spread evenly over the tile's micro-groups: a lone wave hides about five VALU
+  // instructions behind a 32-cycle MFMA (an exponential counts as four) and pays in full for every further one, and with
+  // a whole score element (multiply, exponential, multiply, rounding) beside each MFMA of phases 2 and 3 and nothing
+  // beside those of phases 1 and 4, half of the groups ran at 1.7-2x the MFMA time. So the scores of a block come first
+  // (S: KSTEPS MFMAs, then dP: KSTEPS MFMAs), an element is split into stage A (P = exp2(S c), needs S only) and stage B
+  // (dS = P dP, both rounded to B operands; two elements at a time), and the 32 A and 16 B jobs of a tile fill 48 slots
+  // laid over the groups from the middle of phase 1 to the middle of phase 4 (one slot per group at head_dim 128, two at
+  // 64) in an order that meets every producer and consumer (dK/dV kernel: -12 % cycles, -5.5 % time at head_dim 128):
+  //   half-phase   MFMAs            slots
+  //   0            S0               -
+  //   1            dP0              A0[0..7]
+  //   2            S1               A0[8..15]
+  //   3            dP1              B0[0..7], A1[0..3]
+  //   4            dV0,dK0 (t=0)    B0[8..15], A1[4..7]
+  //   5            dV0,dK0 (t=1)    B1[0..7], A1[8..11]
+  //   6            dV1,dK1 (t=0)    A1[12..15], B1[8..15]
+  //   7            dV1,dK1 (t=1)    -
+  auto tile_body = [&](int j, int buf, auto masked, auto spread) __attribute__((always_inline)) {
     constexpr bool SPREAD = decltype(spread)::value;
+    constexpr int HALF = NMF / 2, NG = 4 * NMF, SPG = 48 / (3 * NMF);      // groups per half-phase / per tile, slots per group
+    static_assert(SPG * 3 * NMF == 48 && kFragAhead <= KSTEPS, "48 slots over the groups of six half-phases");
     const int nbuf = buf == NBUF - 1 ? 0 : buf + 1;
     const int q0t = j * kBwdTile;
-    uint32_t rq[KSTEPS], cq[DBLK][2], rq_next[(kFragAhead + 1) / 2];
+    uint32_t rq[KSTEPS], cq[DBLK][2], rq_next[kFragAhead];
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) { rq[ks] = row_off[ks] + (uint32_t)(buf * TILE_BYTES); asm volatile("" : "+v"(rq[ks])); }
 #pragma unroll
@@ -844,151 +841,125 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
 #pragma unroll
       for (int u = 0; u < 2; ++u) { cq[db][u] = col_off[db][u] + (uint32_t)(buf * TILE_BYTES); asm volatile("" : "+v"(cq[db][u])); }
 #pragma unroll
-    for (int ks = 0; ks < (kFragAhead + 1) / 2; ++ks) { rq_next[ks] = row_off[ks] + (uint32_t)(nbuf * TILE_BYTES); asm volatile("" : "+v"(rq_next[ks])); }
-    // A operand of the tile's MFMA g (phases of NMF)
+    for (int ks = 0; ks < kFragAhead; ++ks) { rq_next[ks] = row_off[ks] + (uint32_t)(nbuf * TILE_BYTES); asm volatile("" : "+v"(rq_next[ks])); }
     auto frag = [&](int g) -> vec8 {
       const int ph = g / NMF, i = g % NMF;
-      return ph < 2 ? scores_frag(rq, ph, i) : grads_frag(cq, ph - 2, i);
+      return ph < 2 ? scores_frag_sd(rq, ph, i) : grads_frag(cq, ph - 2, i);
     };
-    // (past the end of the tile: the first fragments of the next one; read but unused after the last tile)
     auto refill = [&](int g) {
-      fr[g % kFragAhead] = g + kFragAhead < 4 * NMF ? frag(g + kFragAhead) : scores_frag(rq_next, 0, g + kFragAhead - 4 * NMF);
+      fr[g % kFragAhead] = g + kFragAhead < NG ? frag(g + kFragAhead) : scores_frag_sd(rq_next, 0, g + kFragAhead - NG);
     };
-    FO_LDS const float* lse_t = rowvals + buf * kBwdTile;
-    FO_LDS const float* del_t = rowvals + (NBUF + buf) * kBwdTile;
-    f32x4 lv[2];               // LSE of four query rows, fetched one vector ahead
-    // dP = dO V^T - delta comes out of the MFMAs: the accumulator of a block's dP starts from -delta of its 16 rows,
-    // read from LDS straight into the accumulator registers while they are idle (block 1: during phase 1; block 0 of
-    // the next tile: during phase 4, after the hand-over made that tile visible). The block's scores start from
-    // -LSE / scale in the same way, so that QK^T - LSE / scale comes out of the MFMAs.
-    auto start_dp = [&](f32x16& acc, FO_LDS const float* del, int qb) {
+    // an accumulator's start values, straight from LDS into its registers
+    auto start_acc = [&](f32x16& acc, FO_LDS const float* rows, int qb) {
 #pragma unroll
       for (int jv = 0; jv < 4; ++jv) {
-        const f32x4 d4 = *(FO_LDS const f32x4*)(del + 32 * qb + 8 * jv + 4 * hh);
+        const f32x4 d4 = *(FO_LDS const f32x4*)(rows + 32 * qb + 8 * jv + 4 * hh);
 #pragma unroll
         for (int u = 0; u < 4; ++u) acc[4 * jv + u] = d4[u];
       }
     };
-    // score element r of block qb: register r holds query q0t + 32*qb + 4*hh + koff(r), koff(r) = (r & 3) + 8 * (r >> 2);
-    // dead iff key > query or the query is past the end
-    auto element = [&](int qb, int r) {
-      const int jv = r >> 2, u = r & 3;
-      if (!NLSE && u == 0 && jv + 1 < 4) {
-        lv[(jv + 1) & 1] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 8 * (jv + 1) + 4 * hh);
-      }
-      const int koff = u + 8 * jv;
+    float pv[2][16];            // P of a block between its two stages
+    auto stage_a = [&](int qb, int r) {
+      const int koff = (r & 3) + 8 * (r >> 2);
       bool dead = false;
       if constexpr (decltype(masked)::value) {
         const int lim = CAUSAL ? key - (q0t + 32 * qb + 4 * hh) : 0;
         const int lim_end = Sq - (q0t + 32 * qb + 4 * hh);
         dead = koff < lim || koff >= lim_end;
       }
-      // (with NLSE the score accumulator started from -LSE / scale: see start_dp)
-      const float p = dead ? 0.0f : __builtin_amdgcn_exp2f(NLSE ? sacc[qb][r] * c : __builtin_fmaf(sacc[qb][r], c, -lv[jv & 1][u] * kLog2e));
-      const float ds = p * dpacc[qb][r];   // (dP - delta) softmax_scale is applied to the finished dK
-      if (r & 1) {
-        // a finished pair is rounded and pinned to its micro-group: left alone, the compiler moves the multiplication
-        // and the rounding down to the MFMA that reads them, which may not read a register that a VALU instruction
-        // has just written
-        const vec2 p2 = {(T)p_even[qb], (T)p}, ds2 = {(T)ds_even[qb], (T)ds};
-        int pw = __builtin_bit_cast(int, p2), dsw = __builtin_bit_cast(int, ds2);
-        asm volatile("" : "+v"(pw), "+v"(dsw));
-        pf[qb][r >> 3][(r & 7) >> 1] = pw;
-        dsf[qb][r >> 3][(r & 7) >> 1] = dsw;
-      } else {
-        p_even[qb] = p;
-        ds_even[qb] = ds;
-      }
+      pv[qb][r] = dead ? 0.0f : __builtin_amdgcn_exp2f(sacc[qb][r] * c);
     };
-    auto first_rows = [&](int qb) {
-      if (!NLSE) lv[0] = *(FO_LDS const f32x4*)(lse_t + 32 * qb + 4 * hh);
+    auto stage_b = [&](int qb, int r) {          // elements r and r + 1
+      const float ds0 = pv[qb][r] * dpacc[qb][r], ds1 = pv[qb][r + 1] * dpacc[qb][r + 1];
+      const vec2 p2 = {(T)pv[qb][r], (T)pv[qb][r + 1]}, ds2 = {(T)ds0, (T)ds1};
+      int pw = __builtin_bit_cast(int, p2), dsw = __builtin_bit_cast(int, ds2);
+      // (pinned to its micro-group: left alone, the compiler moves the multiplications and the rounding down to the MFMA
+      // that reads them, which may not read a register that a VALU instruction has just written)
+      asm volatile("" : "+v"(pw), "+v"(dsw));
+      pf[qb][r >> 3][(r & 7) >> 1] = pw;
+      dsf[qb][r >> 3][(r & 7) >> 1] = dsw;
     };
-    // ---- phase 1
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < NMF; ++i) {
-      const int g = i;
-      if (i & 1) mfma_scores_vgpr<T>(dpacc[0], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[0], fr[g % kFragAhead], kf[i >> 1], i == 0 && !NLSE);
-      refill(g);
-      if (i == 0) start_dp(dpacc[1], del_t, 1);
-      if (NLSE && i == 1) start_dp(sacc[1], lse_t, 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // ---- phase 2
-    first_rows(0);
-#pragma unroll
-    for (int i = 0; i < NMF; ++i) {
-      const int g = NMF + i;
-      if (i & 1) mfma_scores_vgpr<T>(dpacc[1], fr[g % kFragAhead], vf[i >> 1], false); else mfma_scores_vgpr<T>(sacc[1], fr[g % kFragAhead], kf[i >> 1], i == 0 && !NLSE);
-      refill(g);
-      if (i == 0) scores_fence(sacc[0], dpacc[0]);
-#pragma unroll
-      for (int e = 0; e < EPG; ++e) element(0, i * EPG + e);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // ---- phase 3
-    first_rows(1);
-#pragma unroll
-    for (int i = 0; i < NMF; ++i) {
-      const int g = 2 * NMF + i;
-      const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
-      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, dsf[0][t])); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, pf[0][t]));
-      refill(g);
-      if (i == 0) scores_fence(sacc[1], dpacc[1]);
-#pragma unroll
-      for (int e = 0; e < EPG; ++e) element(1, i * EPG + e);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    auto slot = [&](int s) {
+      const int h = s / 8, u = s % 8;            // half-phase 1 + h, slot u of its eight
+      if (h == 0) stage_a(0, u);
+      else if (h == 1) stage_a(0, 8 + u);
+      else if (h == 2) { if (u < 4) stage_b(0, 2 * u); else stage_a(1, u - 4); }
+      else if (h == 3) { if (u < 4) stage_b(0, 8 + 2 * u); else stage_a(1, u); }
+      else if (h == 4) { if (u < 4) stage_b(1, 2 * u); else stage_a(1, 4 + u); }
+      else { if (u < 4) stage_a(1, 12 + u); else stage_b(1, 8 + 2 * (u - 4)); }
+    };
     const char* next_q = nullptr;
     const char* next_g = nullptr;
     const char* next_rows = nullptr;
     uint32_t next_q_dst = 0;
     FO_LDS char* next_rows_dst = nullptr;
-    if constexpr (SPREAD) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      const int b2 = buf == 0 ? NBUF - 1 : buf - 1, which = wave_s & 1;   // (waves 2 and 3 repeat the row values of waves 0 and 1)
-      next_q = (const char*)(qbase + (int64_t)(j + 2) * kBwdTile * prm.qs[2]);
-      next_g = (const char*)(gbase + (int64_t)(j + 2) * kBwdTile * prm.dos[2]);
-      next_rows = (const char*)((which ? (const float*)prm.delta : lse_src) + (int64_t)bh * Sq + (j + 2) * kBwdTile);
-      next_q_dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem + b2 * TILE_BYTES + wave_s * (TileLaneOffsets<T, D>::N * 1024)));
-      next_rows_dst = (FO_LDS char*)(rowvals + (NBUF * which + b2) * kBwdTile);
-    } else {
-      if (j + 1 < n_qt) hand_over(j);
-    }
-    // ---- phase 4
-    // (two wait states: the paths around the hand-over join here, and the check of the generated code, which follows
-    // no branches, must see that the first MFMA does not read a register written by the VALU instruction before it)
-    asm volatile("s_nop 1");
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < NMF; ++i) {
-      const int g = 3 * NMF + i;
-      const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
-      if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, dsf[1][t])); else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, pf[1][t]));
-      refill(g);
-      if (i == 0) start_dp(dpacc[0], rowvals + (NBUF + nbuf) * kBwdTile, 0);   // (after the last tile: read, unused)
-      if (NLSE && i == 1) start_dp(sacc[0], rowvals + nbuf * kBwdTile, 0);
-      if constexpr (SPREAD) {
-        constexpr int N = TileLaneOffsets<T, D>::N, EVERY = NMF / (2 * N);
-        static_assert(EVERY >= 1 && 2 * N * EVERY == NMF && 2 * N <= 8, "one copy per EVERY micro-groups");
-        auto copy_piece = [&](auto pc) {
-          constexpr int piece = decltype(pc)::value;
-          if constexpr (piece < N) dma16_uniform_base_lds_imm<piece * 1024>(next_q, qlo.off[piece], next_q_dst);
-          else if constexpr (piece < 2 * N) dma16_uniform_base_lds_imm<NBUF * TILE_BYTES + (piece - N) * 1024>(next_g, glo.off[piece - N], next_q_dst);
-        };
-        if (i % EVERY == EVERY - 1) {
-          switch (i / EVERY) {      // (a constant once the loop is unrolled)
-            case 0: copy_piece(std::integral_constant<int, 0>{}); break;
-            case 1: copy_piece(std::integral_constant<int, 1>{}); break;
-            case 2: copy_piece(std::integral_constant<int, 2>{}); break;
-            case 3: copy_piece(std::integral_constant<int, 3>{}); break;
-            case 4: copy_piece(std::integral_constant<int, 4>{}); break;
-            case 5: copy_piece(std::integral_constant<int, 5>{}); break;
-            case 6: copy_piece(std::integral_constant<int, 6>{}); break;
-            default: copy_piece(std::integral_constant<int, 7>{}); break;
-          }
+    for (int g = 0; g < NG; ++g) {
+      const int ph = g / NMF, i = g % NMF;
+      if (g == 3 * NMF) {
+        // the hand-over, between phases 3 and 4 (see hand_over)
+        if constexpr (SPREAD) {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          const int b2 = buf == 0 ? NBUF - 1 : buf - 1, which = wave_s & 1;   // (waves 2 and 3 repeat the row values of waves 0 and 1)
+          next_q = (const char*)(qbase + (int64_t)(j + 2) * kBwdTile * prm.qs[2]);
+          next_g = (const char*)(gbase + (int64_t)(j + 2) * kBwdTile * prm.dos[2]);
+          next_rows = (const char*)((which ? (const float*)prm.delta : (const float*)prm.nlse) + (int64_t)bh * Sq + (j + 2) * kBwdTile);
+          next_q_dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem + b2 * TILE_BYTES + wave_s * (TileLaneOffsets<T, D>::N * 1024)));
+          next_rows_dst = (FO_LDS char*)(rowvals + (NBUF * which + b2) * kBwdTile);
+        } else {
+          if (j + 1 < n_qt) hand_over(j);
         }
-        if (i == 0) dma4_uniform_base(next_rows, lane4, next_rows_dst);
+      }
+      // (two wait states where an MFMA may follow the VALU instruction that wrote its B operand: behind the hand-over,
+      // whose paths join here, and where the last B job of the tile ends right before its first reader)
+      if (g == 3 * NMF || g == 3 * NMF + HALF) asm volatile("s_nop 1");
+      if (ph < 2) {
+        if (i < KSTEPS) mfma_scores_vgpr<T>(sacc[ph], fr[g % kFragAhead], kf[i]);
+        else mfma_scores_vgpr<T>(dpacc[ph], fr[g % kFragAhead], vf[i - KSTEPS]);
+      } else {
+        const int t = i / (2 * DBLK), db = (i >> 1) % DBLK;
+        if (i & 1) mfma_acc_agpr<T>(dkacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, dsf[ph - 2][t]));
+        else mfma_acc_agpr<T>(dvacc[db], fr[g % kFragAhead], __builtin_bit_cast(vec8, pf[ph - 2][t]));
+      }
+      refill(g);
+      // start values of the accumulators while they are idle: block 1 of this tile, block 0 of the next (visible since
+      // the hand-over; after the last tile: read, unused)
+      if (g == 0) start_acc(dpacc[1], rowvals + (NBUF + buf) * kBwdTile, 1);
+      if (g == 1) start_acc(sacc[1], rowvals + buf * kBwdTile, 1);
+      if (g == 3 * NMF) start_acc(dpacc[0], rowvals + (NBUF + nbuf) * kBwdTile, 0);
+      if (g == 3 * NMF + 1) start_acc(sacc[0], rowvals + nbuf * kBwdTile, 0);
+      if constexpr (SPREAD) {
+        if (ph == 3) {
+          constexpr int N = TileLaneOffsets<T, D>::N, EVERY = NMF / (2 * N);
+          static_assert(EVERY >= 1 && 2 * N * EVERY == NMF && 2 * N <= 8, "one copy per EVERY micro-groups");
+          auto copy_piece = [&](auto pc) {
+            constexpr int piece = decltype(pc)::value;
+            if constexpr (piece < N) dma16_uniform_base_lds_imm<piece * 1024>(next_q, qlo.off[piece], next_q_dst);
+            else if constexpr (piece < 2 * N) dma16_uniform_base_lds_imm<NBUF * TILE_BYTES + (piece - N) * 1024>(next_g, glo.off[piece - N], next_q_dst);
+          };
+          if (i % EVERY == EVERY - 1) {
+            switch (i / EVERY) {      // (a constant once the loop is unrolled)
+              case 0: copy_piece(std::integral_constant<int, 0>{}); break;
+              case 1: copy_piece(std::integral_constant<int, 1>{}); break;
+              case 2: copy_piece(std::integral_constant<int, 2>{}); break;
+              case 3: copy_piece(std::integral_constant<int, 3>{}); break;
+              case 4: copy_piece(std::integral_constant<int, 4>{}); break;
+              case 5: copy_piece(std::integral_constant<int, 5>{}); break;
+              case 6: copy_piece(std::integral_constant<int, 6>{}); break;
+              default: copy_piece(std::integral_constant<int, 7>{}); break;
+            }
+          }
+          if (i == 0) dma4_uniform_base(next_rows, lane4, next_rows_dst);
+        }
+      }
+      if (g >= HALF && g < NG - HALF) {
+        // (S of block 0 was finished by the MFMA before this group's: that one and four wait states cover the 11 its
+        // result needs before a VALU instruction may read it; every later first read is several MFMAs behind)
+        if (g == HALF) asm volatile("s_nop 3" : "+v"(sacc[0]));
+#pragma unroll
+        for (int u = 0; u < SPG; ++u) slot((g - HALF) * SPG + u);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1003,22 +974,20 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
   j = ja;
   if (j < n_qt) {
     const int buf = (j - qt0) % NBUF;
-    uint32_t rq0[(kFragAhead + 1) / 2];
+    uint32_t rq0[kFragAhead];
 #pragma unroll
-    for (int ks = 0; ks < (kFragAhead + 1) / 2; ++ks) rq0[ks] = row_off[ks] + (uint32_t)(buf * TILE_BYTES);
+    for (int ks = 0; ks < kFragAhead; ++ks) rq0[ks] = row_off[ks < KSTEPS ? ks : 0] + (uint32_t)(buf * TILE_BYTES);
 #pragma unroll
-    for (int i = 0; i < kFragAhead; ++i) fr[i] = scores_frag(rq0, 0, i);
+    for (int i = 0; i < kFragAhead; ++i) fr[i] = scores_frag_sd(rq0, 0, i);
     // (dP of the first tile's block 0 starts from -delta, as every later one does at the end of the tile before it)
 #pragma unroll
     for (int jv = 0; jv < 4; ++jv) {
       const f32x4 d4 = *(FO_LDS const f32x4*)(rowvals + (NBUF + buf) * kBwdTile + 8 * jv + 4 * hh);
 #pragma unroll
       for (int u = 0; u < 4; ++u) dpacc[0][4 * jv + u] = d4[u];
-      if constexpr (NLSE) {
-        const f32x4 n4 = *(FO_LDS const f32x4*)(rowvals + buf * kBwdTile + 8 * jv + 4 * hh);
+      const f32x4 n4 = *(FO_LDS const f32x4*)(rowvals + buf * kBwdTile + 8 * jv + 4 * hh);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) sacc[0][4 * jv + u] = n4[u];
-      }
+      for (int u = 0; u < 4; ++u) sacc[0][4 * jv + u] = n4[u];
     }
   }
   int buf = j < n_qt ? (j - qt0) % NBUF : 0;
