@@ -670,6 +670,46 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_kernel(const Att
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
+// The softmax-gradient jobs of one tile of the pipelined dK/dV kernel (see its tile_body): 48 slots, slot s = eight per
+// half-phase from the second half of phase 1 on. stage 0 = A of element r (P = exp2(S c)), stage 1 = B of elements r and
+// r + 1 (dS = P dP, both rounded) of query block qb.
+struct SoftmaxGradJob { int stage, qb, r; };
+constexpr SoftmaxGradJob softmax_grad_job(int s) {
+  const int h = s / 8, u = s % 8;
+  if (h == 0) return {0, 0, u};
+  if (h == 1) return {0, 0, 8 + u};
+  if (h == 2) return u < 4 ? SoftmaxGradJob{1, 0, 2 * u} : SoftmaxGradJob{0, 1, u - 4};
+  if (h == 3) return u < 4 ? SoftmaxGradJob{1, 0, 8 + 2 * u} : SoftmaxGradJob{0, 1, u};
+  if (h == 4) return u < 4 ? SoftmaxGradJob{1, 1, 2 * u} : SoftmaxGradJob{0, 1, 4 + u};
+  return u < 4 ? SoftmaxGradJob{0, 1, 12 + u} : SoftmaxGradJob{1, 1, 8 + 2 * (u - 4)};
+}
+// Every element gets each stage once; a job runs behind the MFMA of its group, so stage A of block qb needs a group
+// after the block's last S MFMA, stage B one after its last dP MFMA and a slot after the A jobs of its two elements, and
+// the B operands of elements 8t .. 8t+7 must be complete in a group before the first gradient MFMA that reads them.
+// (The wait states these distances need in instructions are checked on the generated code, fast_ops_amd/asm_lint.py.)
+constexpr bool softmax_grad_jobs_fit(int nmf) {
+  const int half = nmf / 2, ksteps = nmf / 2, spg = 48 / (3 * nmf);
+  if (spg * 3 * nmf != 48) return false;
+  int slot_a[2][16] = {}, slot_b[2][16] = {}, n_a[2][16] = {}, n_b[2][16] = {};
+  for (int s = 0; s < 48; ++s) {
+    const SoftmaxGradJob j = softmax_grad_job(s);
+    if (j.qb < 0 || j.qb > 1 || j.r < 0 || j.r + j.stage > 15) return false;
+    if (j.stage == 0) { slot_a[j.qb][j.r] = s; ++n_a[j.qb][j.r]; }
+    else { slot_b[j.qb][j.r] = slot_b[j.qb][j.r + 1] = s; ++n_b[j.qb][j.r]; ++n_b[j.qb][j.r + 1]; }
+  }
+  for (int qb = 0; qb < 2; ++qb)
+    for (int r = 0; r < 16; ++r) {
+      if (n_a[qb][r] != 1 || n_b[qb][r] != 1) return false;
+      const int ga = half + slot_a[qb][r] / spg, gb = half + slot_b[qb][r] / spg;     // the groups the jobs run in
+      if (ga < qb * nmf + ksteps) return false;                                          // S complete
+      if (gb < (qb + 1) * nmf || slot_b[qb][r] <= slot_a[qb][r]) return false;           // dP complete, P there
+      if (gb >= (2 + qb) * nmf + (r / 8) * half) return false;                           // before its first reader
+    }
+  return true;
+}
+static_assert(softmax_grad_jobs_fit(16) && softmax_grad_jobs_fit(8), "head_dim 128 and 64");
+
+// ---------------------------------------------------------------------------------------------------------------------
 // dK/dV without dropout and bias, as a software pipeline. The accumulators of dK and dV, the K^T and V^T fragments and
 // two blocks of scores leave room for one wave per SIMD only, and a lone wave issues in order: whatever arithmetic sits
 // between two MFMAs keeps the matrix pipe waiting unless it is laid out to run beside them. A 64-query tile is two
@@ -880,13 +920,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
       dsf[qb][r >> 3][(r & 7) >> 1] = dsw;
     };
     auto slot = [&](int s) {
-      const int h = s / 8, u = s % 8;            // half-phase 1 + h, slot u of its eight
-      if (h == 0) stage_a(0, u);
-      else if (h == 1) stage_a(0, 8 + u);
-      else if (h == 2) { if (u < 4) stage_b(0, 2 * u); else stage_a(1, u - 4); }
-      else if (h == 3) { if (u < 4) stage_b(0, 8 + 2 * u); else stage_a(1, u); }
-      else if (h == 4) { if (u < 4) stage_b(1, 2 * u); else stage_a(1, 4 + u); }
-      else { if (u < 4) stage_a(1, 12 + u); else stage_b(1, 8 + 2 * (u - 4)); }
+      const SoftmaxGradJob job = softmax_grad_job(s);      // (s is a constant once the loop is unrolled)
+      if (job.stage == 0) stage_a(job.qb, job.r); else stage_b(job.qb, job.r);
     };
     const char* next_q = nullptr;
     const char* next_g = nullptr;
