@@ -184,11 +184,20 @@ class Lion(Optimizer):
                 if grad is None:
                     continue
                 rec = seen.get(param)
-                if (rec is not None and rec[0] is grad and rec[1] is self.state[param].get("exp_avg")
-                        and rec[3][0] == param.data_ptr() and rec[3][1] == grad.data_ptr() and rec[3][2] == rec[1].data_ptr()):
+                same_p_m = (rec is not None and rec[1] is self.state[param].get("exp_avg")
+                            and rec[3][0] == param.data_ptr() and rec[3][2] == rec[1].data_ptr())
+                if same_p_m and rec[0] is grad and rec[3][1] == grad.data_ptr():
                     # same gradient and momentum objects over the same memory as last step (gradients accumulated in
                     # place): dtypes, devices and layouts cannot have changed, the checks need not be repeated
                     bucket, entry = rec[2], rec[3]
+                elif (same_p_m and grad.dtype == param.dtype and grad.device == param.device and not grad.is_sparse
+                      and grad.shape == param.shape and grad.stride() == param.stride()):
+                    # a new gradient tensor for an unchanged parameter and momentum (zero_grad(set_to_none=True), torch's
+                    # default, makes one every step): only the gradient needs looking at, against the parameter it was
+                    # checked with before
+                    bucket = rec[2]
+                    entry = (rec[3][0], grad.data_ptr(), rec[3][2], rec[3][3])
+                    rec[0], rec[3] = grad, entry
                 else:
                     state = self.state[param]
                     if "exp_avg" not in state:

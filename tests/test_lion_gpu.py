@@ -453,6 +453,39 @@ def test_gradients_accumulated_in_place_and_replaced_between_steps():
     del keep_alive
 
 
+def test_a_bad_gradient_after_good_steps_still_raises():
+    # after the first step only a new gradient tensor is looked at again (torch's zero_grad makes one every step): that
+    # look must still refuse what the full check refuses, and a good one at a new address or as a new object over the
+    # same memory must be used
+    g = torch.Generator().manual_seed(9)
+    p0 = torch.randn(64, 48, generator=g) * 0.02
+    g1, g2, g3 = (torch.randn(64, 48, generator=g) * 0.01 for _ in range(3))
+    prm = torch.nn.Parameter(p0.clone().to(DEV))
+    opt = Lion([prm], **HP)
+    pc, mc = p0.numpy().reshape(-1).copy(), np.zeros(p0.numel(), np.uint16)
+    prm.grad = g1.to(DEV)
+    opt.step()
+    lo.lion_step_c(pc, g1.numpy().reshape(-1).copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    # (a gradient of another dtype never gets this far: torch refuses the assignment)
+    prm.grad = g2.to(DEV).t().contiguous().t()          # right shape, other strides
+    with pytest.raises(RuntimeError, match="contiguous"):
+        opt.step()
+    prm.grad = g2.to(DEV)                                # a good one again, another tensor at another address
+    opt.step()
+    lo.lion_step_c(pc, g2.numpy().reshape(-1).copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    buf = g3.to(DEV)
+    prm.grad = buf.view_as(buf)                          # a new tensor object over memory ...
+    opt.step()
+    lo.lion_step_c(pc, g3.numpy().reshape(-1).copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    buf.copy_(g1.to(DEV))
+    prm.grad = buf.view_as(buf)                          # ... and another one over the same memory with new values
+    opt.step()
+    lo.lion_step_c(pc, g1.numpy().reshape(-1).copy(), mc, HP["lr"], HP["betas"], HP["weight_decay"])
+    torch.cuda.synchronize()
+    assert np.array_equal(_bits32(prm).reshape(-1), pc.view(np.uint32))
+    assert np.array_equal(_bits16(opt.state[prm]["exp_avg"]).reshape(-1), mc)
+
+
 def test_typed_unaligned_views_and_multi_tensor_equivalence():
     # views at odd element offsets take the element-wise path; a multi-tensor launch equals per-tensor launches
     for p_dtype, m_dtype in ((torch.float16, torch.float16), (torch.bfloat16, torch.float32), (torch.float32, torch.float32)):
