@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "libfastops_hip.so")
 
 FO_LION_CHUNK = 8192
 FO_ATTN_BWD_STATIC_ROWS = 1 << 20
+ABI_MAJOR = 2            # fo_version() // 1000 the signatures below belong to
 FO_DTYPE_F16, FO_DTYPE_BF16, FO_DTYPE_F32 = 0, 1, 2
 FO_ATTN_KERNEL_ROWS128, FO_ATTN_KERNEL_ROWS128_EXACT, FO_ATTN_KERNEL_ROWS256_W8, FO_ATTN_KERNEL_ROWS256_W4 = 0, 1, 16, 32
 
@@ -85,6 +86,8 @@ def load() -> ctypes.CDLL:
                 raise FastOpsLibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from e
             fn.restype = restype
             fn.argtypes = argtypes
+        if lib.fo_version() // 1000 != ABI_MAJOR:
+            raise FastOpsLibraryError(f"{LIB_PATH} has ABI version {lib.fo_version()}, this package needs {ABI_MAJOR}xxx; rebuild it")
         _lib = lib
     return _lib
 

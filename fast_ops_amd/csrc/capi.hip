@@ -26,7 +26,7 @@ extern "C" const char* fo_strerror(int status) {
   }
 }
 
-extern "C" int fo_version(void) { return 1000; }
+extern "C" int fo_version(void) { return 2000; }
 
 extern "C" int fo_tune_set(const char* key, int value) {
   if (!key) return FO_ERR_NULL_POINTER;

@@ -41,7 +41,8 @@ enum { FO_DTYPE_F16 = 0, FO_DTYPE_BF16 = 1, FO_DTYPE_F32 = 2 /* Lion entry point
 /* Human-readable text for a status code; never NULL. */
 const char* fo_strerror(int status);
 
-/* Library ABI version: major*1000 + minor. */
+/* Library ABI version: major*1000 + minor. 2000: the workspace of fo_attn_bwd holds two values per query row
+ * ([2, B, H, Sq] fp32; 1000: one), and fo_attn_fwd_kernel / fo_attn_bwd_static_ws exist. */
 int fo_version(void);
 
 /* Tuning hook for benchmarks, profiling and tests: selects a kernel variant or a workgroup order by name

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_strerror():
     lib = _lib.load()
-    assert lib.fo_version() >= 1000
+    assert lib.fo_version() // 1000 == _lib.ABI_MAJOR == 2
     assert _lib.strerror(0) == "ok"
     for code in range(-8, 0):
         assert "unknown" not in _lib.strerror(code)
