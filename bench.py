@@ -1,6 +1,6 @@
 """Benchmark of the two hot paths on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle N] [--path both|attn|lion|copy|clock|ablations]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle N] [--path both|attn|lion|next|copy|clock|power|ablations]
                     [--no-cpu-baseline] [--headline-only]
 
 Prints ONE JSON line. The headline value is the attention forward throughput at B=2 H=16 S=8192 D=128 bf16 causal
@@ -9,7 +9,15 @@ per parameter) is reported in the "lion" object of the same line, each with its 
 this host's cores. Beside them, not part of the headline: the attention backward of the same shape ("attn_bwd"), the
 other three benchmark configurations ("configs": GPT-2-small attention forward, GPT-2-small Lion, fp16 non-causal
 attention forward at B=16 H=32 S=2048 D=128), and the rate of the vendor library's plain bf16 GEMM on random operands
-on the same box ("library_gemm": what MFMA code reaches here at all).
+on the same box ("library_gemm": what MFMA code reaches here at all), and three variations of the headline launch
+("headline_variants": the same shape non-causal, the same causal launch on all-zero operands, and head_dim 64 at
+B=2 H=32 S=8192 causal) with the ratio of the causal time to half the non-causal time.
+
+`--path next` times what lies around the two headline kernels with the same machinery: attention forward, backward and
+forward+backward on the reference's own benchmark matrix (1 x 12 heads x {2048, 4096, 8192} x 128, bf16, with and
+without causal mask, dropout 0.1 and a [B,1,1,S] bias; the reference's published A100 timings are quoted beside them),
+and the fused Lion step at the reference's benchmark sizes (8192 and 8192^2 elements, all-fp16 and all-bf16) and at
+1.3 B parameters for all-bf16 and fp32-momentum tensors.
 
 Every timed section is preceded by a clock-settle phase of --settle launches of the same step (default 100, reported
 under "settle"), which is not part of the W warm-up steps: after idling, the GPU's clocks take a few dozen launches
@@ -56,6 +64,16 @@ def _cpu_model():
     return "unknown"
 
 
+def _host_threads():
+    """Threads for the CPU baselines: the cores this process may run on, at most what OMP_NUM_THREADS allows."""
+    n = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    try:
+        n = min(n, int(os.environ["OMP_NUM_THREADS"]))
+    except (KeyError, ValueError):
+        pass
+    return max(1, n)
+
+
 def _events(n):
     import torch
 
@@ -80,16 +98,25 @@ def _settle(step, launches):
     return {"launches": launches, "ms_first": sum(ms[:k]) / k, "ms_last": sum(ms[-k:]) / k, "ms_max": max(ms)}
 
 
-def _time_steps(step, steps, warmup, settle=0, before_each=None):
+def _time_steps(step, steps, warmup, settle=0, before_each=None, wall_without_events=False):
     """`settle` clock-settle launches, W untimed steps, then K timed steps bracketed by synchronize; per-launch durations
     from HIP events recorded on the stream the kernels are launched on (torch's current stream). `before_each(i)`, if
-    given, runs before timed step i outside its pair of events (fresh inputs for the step)."""
+    given, runs before timed step i outside its pair of events (fresh inputs for the step). With `wall_without_events`
+    the wall time per step comes from K further steps with no events between them (for kernels of a few tens of
+    microseconds, where the two event records per step are a sizeable part of a step)."""
     import torch
 
     info = _settle(step, settle)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    wall_plain = None
+    if wall_without_events:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        wall_plain = (time.perf_counter() - t0) * 1e3 / steps
     starts, ends = _events(steps), _events(steps)
     t0 = time.perf_counter()
     for i in range(steps):
@@ -101,7 +128,8 @@ def _time_steps(step, steps, warmup, settle=0, before_each=None):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     per_launch = [starts[i].elapsed_time(ends[i]) for i in range(steps)]
-    return wall_ms / steps, sum(per_launch) / steps, min(per_launch), info
+    info = dict(info, kernel_ms_median=sorted(per_launch)[steps // 2])
+    return (wall_plain if wall_plain is not None else wall_ms / steps), sum(per_launch) / steps, min(per_launch), info
 
 
 def _attn_inputs(B, H, S, D, dtype, dev, seed=0):
@@ -111,23 +139,52 @@ def _attn_inputs(B, H, S, D, dtype, dev, seed=0):
     return tuple(torch.randn(B, H, S, D, generator=g).to(dtype).to(dev) for _ in range(3)), g
 
 
-def _attn_rate(B, H, S, D, dtype, causal, steps, warmup, settle):
-    """One attention-forward configuration through multi_head_attention: (wall ms per step, kernel ms, min, settle info,
-    FLOPs, which kernel ran)."""
+KERNEL_NAMES = {0: "rows128", 1: "rows128_exact", 16: "rows256_w8", 32: "rows256_w4"}
+
+
+def _attn_rate(B, H, S, D, dtype, causal, steps, warmup, settle, operands="normal", backward=False):
+    """One attention-forward configuration through multi_head_attention: a dict with the wall time per step (steps with
+    no events between them), the kernel time (events), the rate by both and which kernel ran; with `backward`, the same
+    for the backward (dQ + dK/dV launches, five-GEMM FLOP count) under "bwd". `operands`: "normal" (standard normal from
+    the CPU generator, seed 0) or "zero"."""
     import ctypes
 
     import torch
 
     from fast_ops.flash_attention.flash_attention import multi_head_attention
     from fast_ops_amd import _lib
+    from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided
 
-    (q, k, v), _ = _attn_inputs(B, H, S, D, dtype, "cuda:0")
+    (q, k, v), g = _attn_inputs(B, H, S, D, dtype, "cuda:0")
+    if operands == "zero":
+        q, k, v = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
     scale = 1.0 / (D ** 0.5)
     flops = (2.0 if causal else 4.0) * B * H * S * S * D
-    ms_step, ms_kernel, ms_min, info = _time_steps(lambda: multi_head_attention(q, k, v, causal=causal, softmax_scale=scale, return_lse=True), steps, warmup, settle)
+    out = {}
+
+    def fwd():
+        out["o"], out["lse"] = multi_head_attention(q, k, v, causal=causal, softmax_scale=scale, return_lse=True)
+
+    ms_step, ms_kernel, ms_min, info = _time_steps(fwd, steps, warmup, settle, wall_without_events=True)
     I3 = ctypes.c_int64 * 3
     kernel = _lib.load().fo_attn_fwd_kernel(B, H, S, S, D, I3(*k.stride()[:3]), I3(*v.stride()[:3]), int(causal), 0, 0)
-    return ms_step, ms_kernel, ms_min, info, flops, {0: "rows128", 1: "rows128_exact", 16: "rows256_w8", 32: "rows256_w4"}.get(kernel, str(kernel))
+    res = {
+        "workload": f"attention fwd B={B} H={H} S={S} D={D} {'bf16' if dtype == torch.bfloat16 else 'fp16'} {'causal' if causal else 'non-causal'}"
+                    + (", all-zero operands" if operands == "zero" else ""),
+        "ms_per_step": ms_step, "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "achieved": flops / (ms_kernel * 1e-3) / 1e12, "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": flops,
+        "kernel": KERNEL_NAMES.get(kernel, str(kernel)), "kernel_ms_median": info["kernel_ms_median"], "settle": info,
+    }
+    if backward:
+        go = torch.randn(B, H, S, D, generator=g).to(dtype).to("cuda:0")
+        o_fix, lse_fix = out["o"], out["lse"]
+        bflops = 2.5 * flops
+        b_step, b_kernel, b_min, b_info = _time_steps(lambda: attn_bwd_strided(q, k, v, o_fix, lse_fix, go, (0, 1, 2, 3), causal, scale),
+                                                      steps, warmup, settle // 2, wall_without_events=True)
+        res["bwd"] = {"ms_per_step": b_step, "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "kernel_ms_median": b_info["kernel_ms_median"], "value": bflops / (b_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+                      "frac": bflops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": bflops,
+                      "what": "dQ + dK/dV launches of the same shape, FLOPs by the five-GEMM count"}
+    return res
 
 
 def bench_attention(steps, warmup, settle, cpu_baseline, extras):
@@ -189,7 +246,7 @@ def bench_attention(steps, warmup, settle, cpu_baseline, extras):
         # cores, stopped after about 15 s; the rate is that of the slices that were finished
         from oracle.attention_oracle import attention_fwd_oracle
 
-        torch.set_num_threads(os.cpu_count())
+        torch.set_num_threads(_host_threads())
         qc, kc, vc = (t.cpu() for t in (q, k, v))
         attention_fwd_oracle(qc[:1, :1, :1024], kc[:1, :1, :1024], vc[:1, :1, :1024], causal=True, softmax_scale=scale)   # warm-up
         n_sl, t0 = 0, time.perf_counter()
@@ -208,19 +265,25 @@ def bench_attention(steps, warmup, settle, cpu_baseline, extras):
     out.clear()
     torch.cuda.empty_cache()
     if extras:
+        # the headline launch varied one thing at a time, on the same box right after it: what the causal mask costs
+        # against half a non-causal launch, what the operand bits cost (all-zero operands toggle nothing in the
+        # multipliers: the same instruction stream at the clock the power limit then allows), and head_dim 64
+        hv = {
+            "causal": _attn_rate(B, H, S, D, torch.bfloat16, True, steps, warmup, settle),
+            "noncausal": _attn_rate(B, H, S, D, torch.bfloat16, False, steps, warmup, settle),
+            "zero_operands": _attn_rate(B, H, S, D, torch.bfloat16, True, steps, warmup, settle, operands="zero"),
+            "zero_operands_noncausal": _attn_rate(B, H, S, D, torch.bfloat16, False, steps, warmup, settle, operands="zero"),
+            "head_dim_64": _attn_rate(2, 32, 8192, 64, torch.bfloat16, True, steps, warmup, settle),
+        }
+        hv["causal_over_half_noncausal"] = hv["causal"]["kernel_ms_avg"] / (0.5 * hv["noncausal"]["kernel_ms_avg"])
+        res["headline_variants"] = hv
+        torch.cuda.empty_cache()
         # the other attention configurations: report only
-        res["configs"] = {}
-        for name, (b_, h_, s_, d_, dt_, causal_) in {
-            "2_attn_fwd_gpt2_small": (8, 12, 1024, 64, torch.bfloat16, True),
-            "5a_attn_fwd_throughput": (16, 32, 2048, 128, torch.float16, False),
-        }.items():
-            c_step, c_kernel, c_min, c_info, c_flops, c_k = _attn_rate(b_, h_, s_, d_, dt_, causal_, steps, warmup, settle)
-            res["configs"][name] = {
-                "workload": f"attention fwd B={b_} H={h_} S={s_} D={d_} {'bf16' if dt_ == torch.bfloat16 else 'fp16'} {'causal' if causal_ else 'non-causal'}",
-                "ms_per_step": c_step, "kernel_ms_avg": c_kernel, "kernel_ms_min": c_min, "value": c_flops / (c_step * 1e-3) / 1e12, "unit": "TFLOP/s",
-                "frac": c_flops / (c_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": c_flops, "kernel": c_k, "settle": c_info,
-            }
-            torch.cuda.empty_cache()
+        res["configs"] = {
+            "2_attn_fwd_gpt2_small": _attn_rate(8, 12, 1024, 64, torch.bfloat16, True, steps, warmup, settle, backward=True),
+            "5a_attn_fwd_throughput": _attn_rate(16, 32, 2048, 128, torch.float16, False, steps, warmup, settle, backward=True),
+        }
+        torch.cuda.empty_cache()
     return res
 
 
@@ -288,9 +351,52 @@ def bench_lion(steps, warmup, settle, cpu_baseline, extras):
             "note": "ms_per_step includes copying the fresh gradients; value and frac are from the events around each of the 10 steps "
                     "alone, which the GPU reaches before the host has issued the step, so they contain the host's time to issue it",
         }
-        del opt, params, fresh
-        torch.cuda.empty_cache()
+        del opt, fresh, views, grads
+        # the same parameter set in torch's default training loop: backward (autograd makes new gradient tensors), step(),
+        # zero_grad() (set_to_none=True frees them). Host time of step() by the host's clock, kernel time by events around
+        # the step, how often the chunk table had to be rebuilt, and what stays allocated after zero_grad().
+        for p in params:
+            p.grad = None
+        from fast_ops.lion.lion_optimizer import Lion
 
+        opt = Lion(params, **LION_HP)
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        other0 = torch.cuda.memory_allocated() - sum(p.numel() * 4 for p in params)    # whatever else this process holds
+        w = (torch.randn(n_small, generator=torch.Generator().manual_seed(7)) * 1e-2).to(dev)
+        wv, at = [], 0
+        for p in params:
+            wv.append(w[at:at + p.numel()].view(p.shape))
+            at += p.numel()
+        host_us, kern_ms, held = [], [], []
+        n_loop, skip = 30, 10
+        ev = _events(2 * n_loop)
+        rebuilds0 = None
+        for it in range(n_loop):
+            loss = sum([(p * v_).sum() for p, v_ in zip(params, wv)])
+            loss.backward()
+            del loss
+            torch.cuda.synchronize()
+            if it == skip:
+                rebuilds0 = opt.table_rebuilds
+            ev[2 * it].record()
+            t0 = time.perf_counter()
+            opt.step()
+            host_us.append((time.perf_counter() - t0) * 1e6)
+            ev[2 * it + 1].record()
+            opt.zero_grad()
+            torch.cuda.synchronize()
+            kern_ms.append(ev[2 * it].elapsed_time(ev[2 * it + 1]))
+            held.append(torch.cuda.memory_allocated() - other0 - n_small * (4 + 2 + 4))   # parameters, bf16 momenta, w
+        hs, ks = sorted(host_us[skip:]), sorted(kern_ms[skip:])
+        res_small["training_loop"] = {
+            "what": "backward (autograd), step(), zero_grad() with set_to_none=True; figures over the last 20 of 30 iterations",
+            "host_us_step_median": hs[len(hs) // 2], "host_us_step_min": hs[0], "step_ms_by_events_median": ks[len(ks) // 2],
+            "table_rebuilds": opt.table_rebuilds - rebuilds0, "table_rebuilds_first_iterations": rebuilds0,
+            "bytes_allocated_after_zero_grad_beyond_params_momenta_inputs": max(held[skip:]), "bytes_of_one_gradient_set": 4 * n_small,
+        }
+        del opt, params, w, wv
+        torch.cuda.empty_cache()
     shapes = LION_LARGE_SHAPES
     n_params = sum(a * b for a, b in shapes)
     params, opt = _lion_setup(shapes, dev)
@@ -312,7 +418,7 @@ def bench_lion(steps, warmup, settle, cpu_baseline, extras):
         # cores, 3 steps
         from oracle.lion_oracle import lion_step_torch
 
-        torch.set_num_threads(os.cpu_count())
+        torch.set_num_threads(_host_threads())
         n_t = 8
         ps = [params[i].detach().cpu().clone() for i in range(n_t)]
         gs = [params[i].grad.cpu().clone() for i in range(n_t)]
@@ -331,6 +437,109 @@ def bench_lion(steps, warmup, settle, cpu_baseline, extras):
     del opt, params
     torch.cuda.empty_cache()
     return res
+
+
+# The reference's published timings on an A100 (fast_ops/flash_attention/README.md:76-175, column "Triton": its working
+# implementation; fast_ops/lion/README.md:29-35, column "ours"), in microseconds, quoted beside this build's figures as
+# context - other hardware, not a baseline of this benchmark. Keys: (seq_len, dropout_p, bias, causal) -> (fwd, bwd, fwd+bwd).
+REF_A100_TRITON_US = {
+    (2048, 0.0, 0, 0): (258.2, 1020.9, 1354.6), (2048, 0.0, 0, 1): (188.7, 730.1, 938.6), (2048, 0.1, 0, 0): (283.4, 826.7, 1132.7),
+    (2048, 0.1, 0, 1): (230.7, 832.7, 1025.9), (2048, 0.0, 1, 0): (232.7, 870.6, 1129.0), (2048, 0.0, 1, 1): (192.1, 989.8, 1258.1),
+    (2048, 0.1, 1, 0): (286.4, 857.1, 1161.1), (2048, 0.1, 1, 1): (233.0, 875.8, 1191.0),
+    (4096, 0.0, 0, 0): (926.5, 2931.5, 3886.3), (4096, 0.0, 0, 1): (548.9, 2035.1, 2609.7), (4096, 0.1, 0, 0): (1102.2, 2965.1, 4084.2),
+    (4096, 0.1, 0, 1): (674.3, 1847.9, 2539.7), (4096, 0.0, 1, 0): (901.7, 3130.8, 4055.6), (4096, 0.0, 1, 1): (565.9, 2453.2, 3036.3),
+    (4096, 0.1, 1, 0): (1112.0, 3058.4, 4186.3), (4096, 0.1, 1, 1): (681.9, 1954.6, 2660.6),
+    (8192, 0.0, 0, 0): (3415.7, 11207.1, 14681.4), (8192, 0.0, 0, 1): (1788.7, 6593.9, 8263.1), (8192, 0.1, 0, 0): (4244.1, 11320.8, 15619.1),
+    (8192, 0.1, 0, 1): (2230.5, 5854.1, 8129.3), (8192, 0.0, 1, 0): (3411.3, 12037.3, 15479.7), (8192, 0.0, 1, 1): (1847.7, 7640.0, 9533.0),
+    (8192, 0.1, 1, 0): (4215.3, 11619.2, 15894.8), (8192, 0.1, 1, 1): (2258.7, 6188.9, 8485.7),
+}
+REF_A100_LION_US = {(8192, "fp16"): 25.1, (8192, "bf16"): 25.0, (8192 ** 2, "fp16"): 651.9, (8192 ** 2, "bf16"): 710.1}
+
+
+def bench_next(steps, warmup, settle):
+    """What lies around the two headline kernels, timed with the same machinery. Attention: the reference's benchmark
+    matrix (benchmarks/benchmark_flash_attention.py:195-209 and the table of fast_ops/flash_attention/README.md:76-175):
+    [1, S, 12, 128] bf16 tensors through flash_attn, S in {2048, 4096, 8192}, causal or not, dropout 0 / 0.1, no bias / a
+    [1, 1, 1, S] bias; forward (no autograd), backward alone (the two backward launches on saved O and LSE) and forward +
+    backward through autograd. Lion: benchmarks/benchmark_lion.py:10-16 (one tensor of 8192 or 8192^2 elements, all-fp16
+    or all-bf16, lr 1e-4, betas (0.9, 0.99), weight decay 0.1) and the 1.3 B-parameter set with all-bf16 tensors and with
+    fp32 parameters + fp32 momentum."""
+    import math
+
+    import torch
+
+    from fast_ops.lion.lion_optimizer import Lion
+    from fast_ops_amd.flash_attention.flash_attention import attn_bwd_strided, attn_fwd_strided, flash_attn, next_dropout_state
+
+    dev = "cuda:0"
+    B, H, D = 1, 12, 128
+    dims = (0, 2, 1, 3)
+    rows = []
+    g = torch.Generator().manual_seed(0)
+    for S in (2048, 4096, 8192):
+        q, k, v, go = (torch.randn(B, S, H, D, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
+        bias_t = torch.randn(B, 1, 1, S, generator=g).to(torch.bfloat16).to(dev)
+        for has_bias in (0, 1):
+            for p_drop in (0.0, 0.1):
+                for causal in (0, 1):
+                    bias = bias_t if has_bias else None
+                    flops = (2.0 if causal else 4.0) * B * H * S * S * D
+                    f_step, f_kernel, f_min, _ = _time_steps(lambda: flash_attn(q, k, v, bias, bool(causal), p_drop), steps, warmup, settle,
+                                                             wall_without_events=True)
+                    drop = None if p_drop == 0.0 else (p_drop,) + next_dropout_state(B * H * S * S)
+                    o, lse = attn_fwd_strided(q, k, v, dims, bool(causal), None, drop, bias)
+                    b_step, b_kernel, b_min, _ = _time_steps(lambda: attn_bwd_strided(q, k, v, o, lse, go, dims, bool(causal), None, drop, bias),
+                                                             steps, warmup, settle // 2, wall_without_events=True)
+                    qr, kr, vr = (t.detach().requires_grad_(True) for t in (q, k, v))
+
+                    def both():
+                        flash_attn(qr, kr, vr, bias, bool(causal), p_drop).backward(go)
+                        qr.grad = kr.grad = vr.grad = None
+
+                    fb_step, fb_kernel, fb_min, _ = _time_steps(both, steps, warmup, settle // 2, wall_without_events=True)
+                    ref = REF_A100_TRITON_US[(S, p_drop, has_bias, causal)]
+                    rows.append({
+                        "shape": f"({B},{H},{S},{D})", "dropout_p": p_drop, "bias": has_bias, "causal": causal,
+                        "fwd_us": f_kernel * 1e3, "fwd_us_wall": f_step * 1e3, "fwd_tflops": flops / (f_kernel * 1e-3) / 1e12,
+                        "bwd_us": b_kernel * 1e3, "bwd_us_wall": b_step * 1e3, "bwd_tflops": 2.5 * flops / (b_kernel * 1e-3) / 1e12,
+                        "fwd_bwd_us": fb_kernel * 1e3, "fwd_bwd_us_wall": fb_step * 1e3,
+                        "reference_a100_triton_us": {"fwd": ref[0], "bwd": ref[1], "fwd_bwd": ref[2]},
+                    })
+                    del o, lse, qr, kr, vr
+        del q, k, v, go, bias_t
+        torch.cuda.empty_cache()
+    hp = dict(lr=1e-4, betas=(0.9, 0.99), weight_decay=0.1)
+    lion_rows = []
+    for size in (8192, 8192 ** 2):
+        for dt, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+            prm = torch.nn.Parameter(torch.randn(size, generator=g).to(dt).to(dev))
+            prm.grad = torch.randn(size, generator=g).to(dt).to(dev)
+            opt = Lion([prm], **hp)
+            l_step, l_kernel, l_min, _ = _time_steps(opt.step, steps, warmup, settle, wall_without_events=True)
+            lion_rows.append({
+                "elements": size, "dtypes": f"all {name}", "bytes_per_element": 10, "step_us": l_kernel * 1e3, "step_us_wall": l_step * 1e3,
+                "gb_per_s": 10.0 * size / (l_kernel * 1e-3) / 1e9, "frac_of_hbm_peak": 10.0 * size / (l_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                "reference_a100_us": REF_A100_LION_US[(size, name)],
+            })
+            del opt, prm
+    torch.cuda.empty_cache()
+    n_params = sum(a * b for a, b in LION_LARGE_SHAPES)
+    for p_dt, m_dt, name, nbytes in ((torch.bfloat16, torch.bfloat16, "all bf16", 10), (torch.float32, torch.float32, "fp32 parameters and gradients, fp32 momentum", 20),
+                                     (torch.float32, torch.bfloat16, "fp32 parameters and gradients, bf16 momentum (the headline kernel)", 16)):
+        params = [torch.nn.Parameter(torch.empty(sh, dtype=p_dt, device=dev).normal_(0, 0.02)) for sh in LION_LARGE_SHAPES]
+        for prm in params:
+            prm.grad = torch.empty_like(prm).normal_(0, 1e-2)
+        opt = Lion(params, exp_avg_dtype=m_dt, **hp)
+        l_step, l_kernel, l_min, _ = _time_steps(opt.step, min(steps, 50), warmup, min(settle, 20))
+        lion_rows.append({
+            "elements": n_params, "dtypes": name, "bytes_per_element": nbytes, "step_us": l_kernel * 1e3, "step_us_wall": l_step * 1e3,
+            "gb_per_s": float(nbytes) * n_params / (l_kernel * 1e-3) / 1e9, "frac_of_hbm_peak": float(nbytes) * n_params / (l_kernel * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        })
+        del opt, params
+        torch.cuda.empty_cache()
+    return {"path": "next", "attention_reference_matrix": rows, "lion": lion_rows,
+            "note": "times from HIP events around each call (mean over the timed steps); *_wall = host wall clock per call over as many calls "
+                    "without events; reference figures are the reference's own published A100 timings, quoted for context"}
 
 
 def bench_clock(steps, warmup, settle):
@@ -493,8 +702,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle", type=int, default=100,
                     help="clock-settle launches ahead of the warm-up of every timed section (reported, not counted as warm-up)")
-    ap.add_argument("--path", choices=["both", "attn", "lion", "copy", "clock", "power", "ablations"], default="both",
-                    help="copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
+    ap.add_argument("--path", choices=["both", "attn", "lion", "next", "copy", "clock", "power", "ablations"], default="both",
+                    help="next: the reference's benchmark matrix (forward, backward, forward+backward with bias and dropout) and the "
+                         "typed Lion kernels; copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
                          "clock: the attention kernel against the number of busy CUs and the operand bits, with the library GEMM; "
                          "power: socket power (the driver's sensor) while each kernel loops for 3 s; "
                          "ablations: the attention kernel with parts left out (needs a build with --ablations)")
@@ -524,6 +734,9 @@ def main():
         return
     if args.path == "clock":
         print(json.dumps(bench_clock(args.steps, args.warmup, args.settle)))
+        return
+    if args.path == "next":
+        print(json.dumps(bench_next(args.steps, args.warmup, args.settle)))
         return
     if args.path == "power":
         print(json.dumps({"path": "power", **bench_power(3.0)}))
@@ -556,6 +769,8 @@ def main():
         line["attn_bwd"] = attn["bwd"]
     if attn is not None and "library_gemm" in attn:
         line["library_gemm"] = attn["library_gemm"]
+    if attn is not None and "headline_variants" in attn:
+        line["headline_variants"] = attn["headline_variants"]
     configs = {}
     for part in (attn, lion):
         if part is not None:
