@@ -17,7 +17,7 @@ FO_LION_CHUNK = 8192
 FO_ATTN_BWD_STATIC_ROWS = 1 << 20
 ABI_MAJOR = 2            # fo_version() // 1000 the signatures below belong to
 FO_DTYPE_F16, FO_DTYPE_BF16, FO_DTYPE_F32 = 0, 1, 2
-FO_ATTN_KERNEL_ROWS128, FO_ATTN_KERNEL_ROWS128_EXACT, FO_ATTN_KERNEL_ROWS256_W8, FO_ATTN_KERNEL_ROWS256_W4 = 0, 1, 16, 32
+FO_ATTN_KERNEL_ROWS128, FO_ATTN_KERNEL_ROWS128_EXACT, FO_ATTN_KERNEL_ROWS128_PIPE, FO_ATTN_KERNEL_ROWS256_W8, FO_ATTN_KERNEL_ROWS256_W4 = 0, 1, 8, 16, 32
 
 
 class FoLionConsts(ctypes.Structure):

@@ -133,9 +133,11 @@ def lint_function(lines: Iterable[str], name: str) -> List[str]:
 
 
 def lint_file(path: str, name_filter: str) -> List[str]:
-    """Lints every function of the assembly file whose symbol matches the regular expression `name_filter`."""
+    """Lints every function of the assembly file whose symbol matches the regular expression `name_filter`. A filter
+    that matches no function is reported as a problem: a check that looked at nothing must not read as a pass."""
     pat = re.compile(name_filter)
     problems: List[str] = []
+    matched = 0
     cur_name, cur_lines = None, []
     with open(path) as f:
         for raw in f:
@@ -144,12 +146,15 @@ def lint_file(path: str, name_filter: str) -> List[str]:
                 head = s.split(";")[0].rstrip()
                 if head.endswith(":") and not head.startswith((".", " ", "\t")) and pat.search(head):
                     cur_name, cur_lines = head[:-1], []
+                    matched += 1
             else:
                 if s.startswith(".Lfunc_end"):
                     problems += lint_function(cur_lines, cur_name)
                     cur_name = None
                 else:
                     cur_lines.append(s)
+    if matched == 0:
+        problems.append(f"{path}: no function matches {name_filter!r}")
     return problems
 
 

@@ -47,7 +47,8 @@ SOURCES = {
 }
 # sources whose generated assembly is checked by asm_lint: source -> regular expression of the kernel symbols to check
 # (the instantiations with a non-zero last template argument are timing experiments with wrong results by design)
-ASM_LINTED = {"attn_fwd.hip": r"attn_fwd_wide_kernel.*ELi0EEEvNS_10AttnParamsE", "attn_bwd.hip": r"attn_bwd_dkdv_pipe_kernel"}
+# (attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM>: DBG is the last but one)
+ASM_LINTED = {"attn_fwd.hip": r"attn_fwd_wide_kernel.*ELi0ELi\d+EEEvNS_10AttnParamsE", "attn_bwd.hip": r"attn_bwd_dkdv_pipe_kernel"}
 
 
 def _hipcc() -> str:
@@ -90,21 +91,34 @@ def _compile_one(hipcc: str, src: str, extra: list, force: bool, verbose: bool) 
     # the device assembly, which is then checked for the hazards the compiler cannot see inside an asm statement. If the
     # check finds one, compile again with the wait states.
     from .asm_lint import lint_file, lint_m0_file
-    _run_hipcc([hipcc] + COMMON_FLAGS + extra + ["-DFO_MFMA_NOPS=0", "-save-temps=obj", "-c", src_path, "-o", obj], src, verbose)
-    asm = os.path.join(OBJ_DIR, f"{stem}-hip-amdgcn-amd-amdhsa-{ARCH}.s")
-    problems = lint_file(asm, ASM_LINTED[src]) if os.path.exists(asm) else [f"{asm} was not produced"]
-    # the direct-to-LDS copies are inline assembly too: M0 written and read back to back has no fallback build, it is
-    # an error in the source
-    m0_problems = lint_m0_file(asm) if os.path.exists(asm) else []
-    for f in os.listdir(OBJ_DIR):           # the other intermediate files are large and of no further use
-        if f.startswith(stem + "-") or f.startswith(stem + ".hip-"):
-            os.remove(os.path.join(OBJ_DIR, f))
-    if m0_problems:
-        raise RuntimeError(f"{src}: {len(m0_problems)} LDS-DMA instruction(s) issued directly after a write of M0, e.g. {m0_problems[0]}")
+
+    def compile_and_lint(nops: int):
+        _run_hipcc([hipcc] + COMMON_FLAGS + extra + [f"-DFO_MFMA_NOPS={nops}", "-save-temps=obj", "-c", src_path, "-o", obj], src, verbose)
+        asm = os.path.join(OBJ_DIR, f"{stem}-hip-amdgcn-amd-amdhsa-{ARCH}.s")
+        if not os.path.exists(asm):
+            raise RuntimeError(f"{src}: {asm} was not produced, the generated assembly cannot be checked")
+        problems = lint_file(asm, ASM_LINTED[src])
+        # the direct-to-LDS copies are inline assembly too: M0 written and read back to back has no fallback build, it is
+        # an error in the source
+        m0_problems = lint_m0_file(asm)
+        for f in os.listdir(OBJ_DIR):           # the other intermediate files are large and of no further use
+            if f.startswith(stem + "-") or f.startswith(stem + ".hip-"):
+                os.remove(os.path.join(OBJ_DIR, f))
+        if m0_problems:
+            raise RuntimeError(f"{src}: {len(m0_problems)} LDS-DMA instruction(s) issued directly after a write of M0, e.g. {m0_problems[0]}")
+        if any("no function matches" in p for p in problems):
+            raise RuntimeError(f"{src}: the assembly check found no kernel to look at ({ASM_LINTED[src]!r} is out of date)")
+        return problems
+
+    problems = compile_and_lint(0)
     if problems:
         if verbose:
             print(f"{src}: {len(problems)} MFMA hazard(s) without wait states, e.g. {problems[0]}\n  -> compiling with wait states", flush=True)
-        _run_hipcc([hipcc] + COMMON_FLAGS + extra + ["-DFO_MFMA_NOPS=1", "-c", src_path, "-o", obj], src, verbose)
+        # the object that is linked is the one that was checked: the build with wait states goes through the same check
+        # (a hazard that remains there is an error in the source)
+        problems = compile_and_lint(1)
+        if problems:
+            raise RuntimeError(f"{src}: {len(problems)} MFMA hazard(s) remain with wait states in front of every MFMA, e.g. {problems[0]}")
     elif verbose:
         print(f"{src}: inline-assembly MFMAs checked, no hazard", flush=True)
     return obj

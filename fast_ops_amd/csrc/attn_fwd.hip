@@ -477,8 +477,9 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 #ifndef FO_MFMA_NOPS
 #define FO_MFMA_NOPS 1
 #endif
-// Three layout choices of the 256-row kernel, each a bit mask over QB (1: eight waves x 32 rows, 2: four waves x 64 rows),
-// kept as macros so that a build can measure them against each other:
+// Three layout choices of the pipelined kernel, each a bit mask over its forms (1: 256 rows as eight waves x 32 rows,
+// 2: 256 rows as four waves x 64 rows, 4: 128 rows as four waves x 32 rows), kept as macros so that a build can measure
+// them against each other:
 // FO_PIN_MFMA  the MFMA of a micro-group is fenced to be its first instruction. A lone wave per SIMD issues in order: left
 //              to the compiler, the MFMAs of two neighbouring groups end up back to back with all the other work after
 //              them, and the second one stalls the wave for the 28 cycles the matrix pipe is still busy. Four-wave form:
@@ -495,7 +496,7 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 #define FO_STAGGER 0
 #endif
 #ifndef FO_SPREAD
-#define FO_SPREAD 3
+#define FO_SPREAD 7
 #endif
 template <typename T, bool NOP> struct AsmMfma;
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -558,9 +559,15 @@ __device__ __forceinline__ void scale_acc(f32x16& acc, float a) {
 // workgroups per head of the wide kernel
 __host__ __device__ inline int wide_items(int n_qblk, bool causal) { return causal ? (n_qblk + 1) / 2 : n_qblk; }
 
-template <typename T, int D, bool CAUSAL, int QB, int DBG>
-__global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel(const AttnParams prm) {
-  constexpr int kWideWaves = kWideBM / (32 * QB);
+template <typename T, int D, bool CAUSAL, int QB, int DBG, int BM = kWideBM>
+__global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 128) ? 1 : 2) attn_fwd_wide_kernel(const AttnParams prm) {
+  // BM = 256: the form described above. BM = 128 (QB = 1): the same pipeline with four waves x 32 rows, one query block
+  // per workgroup in the 128-row kernel's order (heaviest causal blocks first), for shapes that give the chip too few
+  // 256-row workgroups: a workgroup's time per key tile is what bounds those, and this pipeline's is less than half the
+  // plain 128-row kernel's (which computes S, the softmax and P V of a tile one after the other).
+  static_assert(BM == kWideBM || (BM == kBM && QB == 1), "forms of the pipelined kernel");
+  constexpr bool PAIRED = CAUSAL && BM == kWideBM;   // a causal workgroup takes two query blocks
+  constexpr int kWideWaves = BM / (32 * QB);
   typedef AsmMfma<T, true> Mfma;                  // outside the loops: always with wait states
   typedef __attribute__((ext_vector_type(2))) T vec2;
   constexpr int ROW_BYTES = D * 2;
@@ -574,7 +581,8 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   static_assert(VFRAGS == KSTEPS && DMA_PER_WAVE >= 1 && KSTEPS >= 4, "tile shape");
   // Who issues the copies of a tile: every wave its own blocks (ISSUERS == 1), or the two waves of a SIMD in turn, each
   // the blocks of both (ISSUERS == 2: while one wave is held up at the memory pipe the other has the SIMD to itself).
-  constexpr int ISSUERS = (FO_STAGGER && QB == 1 && !(FO_SPREAD & QB)) ? 2 : 1;
+  constexpr int FORM = BM == kWideBM ? QB : 4;   // bit of this form in the FO_PIN_MFMA / FO_SPREAD masks
+  constexpr int ISSUERS = (FO_STAGGER && BM == kWideBM && QB == 1 && !(FO_SPREAD & FORM)) ? 2 : 1;
   constexpr int NBLK = DMA_PER_WAVE * ISSUERS;          // blocks a wave copies per matrix when it is its turn
 
   extern __shared__ __attribute__((aligned(1024))) char smem_raw[];
@@ -587,22 +595,33 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
 
   // A causal workgroup takes two query blocks, one after the other: block n-1-i (the heaviest left) and block i, so
   // that every workgroup has the same amount of work (n+1 tiles' worth) whatever i is. Non-causal: one block each.
+  // (BM = 128: one block each, causal or not, heaviest blocks first as in attn_fwd_kernel.)
   const int n_bh = prm.B * prm.H;
-  const int n_items = wide_items(prm.n_qblk, CAUSAL);
+  const int n_items = PAIRED ? wide_items(prm.n_qblk, true) : prm.n_qblk;
   int bh, item;
   {
     const int id = blockIdx.x;
     if ((n_bh & 7) == 0) {
-      const int x = id & 7, j = id >> 3;          // XCD, position in that XCD's list: one head after the other
-      bh = x + 8 * (j / n_items);
-      item = j % n_items;
+      const int x = id & 7, j = id >> 3;          // XCD, position in that XCD's list
+      if (BM != kWideBM && CAUSAL && prm.heavy_first > 0) {
+        // groups of heavy_first heads; inside a group the heaviest query blocks of all its heads first
+        const int n_bh_x = n_bh >> 3, per_group = prm.heavy_first * prm.n_qblk;
+        const int grp = j / per_group, r = j - grp * per_group;
+        const int heads = min(prm.heavy_first, n_bh_x - grp * prm.heavy_first);
+        bh = x + 8 * (grp * prm.heavy_first + r % heads);
+        item = r / heads;
+      } else {
+        bh = x + 8 * (j / n_items);               // one head after the other
+        item = j % n_items;
+      }
     } else {
       bh = id % n_bh;
       item = id / n_bh;
     }
+    if (BM != kWideBM && CAUSAL) item = prm.n_qblk - 1 - item;   // heaviest first
   }
   const int b = bh / prm.H, h = bh % prm.H;
-  const int n_pass = (CAUSAL && prm.n_qblk - 1 - item != item) ? 2 : 1;
+  const int n_pass = (PAIRED && prm.n_qblk - 1 - item != item) ? 2 : 1;
   // Q^T fragments (B operand of S^T = K Q^T), QB blocks of 32 query rows, of the query block a pass works on. The
   // second pass's are fetched when the first pass has computed its last scores, so that they arrive while it
   // normalises and writes its O.
@@ -611,20 +630,20 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
     const T* qb_base = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      const int qrow = min(for_qblk * kWideBM + wave_s * 32 * QB + 32 * qb + l32, prm.Sq - 1);
+      const int qrow = min(for_qblk * BM + wave_s * 32 * QB + 32 * qb + l32, prm.Sq - 1);
       const T* qp = qb_base + (int64_t)qrow * prm.qs[2] + 8 * hh;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) qf[qb][ks] = *(const i32x4*)(qp + 16 * ks);
     }
   };
   for (int pass = 0; pass < n_pass; ++pass) {
-  const int qblk = CAUSAL ? (pass == 0 ? prm.n_qblk - 1 - item : item) : item;
+  const int qblk = PAIRED ? (pass == 0 ? prm.n_qblk - 1 - item : item) : item;
   if (pass > 0) {
     // the other waves may still be reading the rings, and this wave's stores of O still count as memory operations in flight
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
-  const int q0 = qblk * kWideBM;
+  const int q0 = qblk * BM;
   const int q0w = q0 + wave_s * 32 * QB;
   const int Sq = prm.Sq, Sk = prm.Sk;
   const T* __restrict__ kbase = (const T*)prm.k + b * prm.ks[0] + h * prm.ks[1];
@@ -632,7 +651,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
 
   int n_tiles, n_w;                       // tiles the workgroup walks / tiles in which this wave has unmasked keys
   if constexpr (CAUSAL) {
-    n_tiles = (min(Sk, q0 + kWideBM) + kBN - 1) / kBN;
+    n_tiles = (min(Sk, q0 + BM) + kBN - 1) / kBN;
     n_w = min(n_tiles, (q0w + 32 * QB - 1) / kBN + 1);
   } else {
     n_tiles = (Sk + kBN - 1) / kBN;
@@ -744,7 +763,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   i32x4 PF[2][QB][2];          // P of sub-tile s: PF[s & 1][qb][16-key step]
   // issue the copies of a tile between the MFMAs of its steps instead of at its top (in the loop of unmasked tiles whose
   // copies are all whole tiles; everywhere else they go out at the top)
-  constexpr bool SPREAD_DMA = (DBG & 8) != 0 || (FO_SPREAD & QB) != 0;
+  constexpr bool SPREAD_DMA = (DBG & 8) != 0 || (FO_SPREAD & FORM) != 0;
   constexpr int RD = QB == 2 ? 4 : 2;       // must divide the number of fragments of a sub-tile
   static_assert(KSTEPS % RD == 0, "fragment ring");
   i32x4 KF[RD], VF[RD];        // LDS fragment rings, refilled RD fragments ahead of use
@@ -834,11 +853,11 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
       } else if (is_qk) {
         if (f == 0) Mfma::v_init_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
         else Mfma::v_acc_ba(S[P ^ 1][qb], KF[f % RD], qf[qb][f]);
-        if (FO_PIN_MFMA & QB) __builtin_amdgcn_sched_barrier(0);
+        if (FO_PIN_MFMA & FORM) __builtin_amdgcn_sched_barrier(0);
         if (qb == QB - 1 && !(DBG & 4)) KF[f % RD] = (f + RD < KSTEPS) ? k_frag(kb1, f + RD) : k_frag(kb2, f + RD - KSTEPS);
       } else {
         Mfma::a_acc(oacc[f % DBLK][qb], VF[f % RD], PF[P ^ 1][qb][f / DBLK]);
-        if (FO_PIN_MFMA & QB) __builtin_amdgcn_sched_barrier(0);
+        if (FO_PIN_MFMA & FORM) __builtin_amdgcn_sched_barrier(0);
         if (qb == QB - 1 && !(DBG & 4)) VF[f % RD] = (f + RD < VFRAGS) ? v_frag(vb0, f + RD) : v_frag(vb1, f + RD - VFRAGS);
       }
       if constexpr (!HAS_PV) {
@@ -1045,7 +1064,7 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   // tiles in which this wave has nothing to do (causal): keep feeding the workgroup's rings
   for (; j < n_tiles; ++j) tile_top(j);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (CAUSAL && pass + 1 < n_pass) load_q(item);   // (the second pass works on query block `item`)
+  if (PAIRED && pass + 1 < n_pass) load_q(item);   // (the second pass works on query block `item`)
 
   // ---- epilogue: normalise, write O and LSE
 #pragma unroll
@@ -1092,15 +1111,41 @@ __global__ void __launch_bounds__(kWideBM / (32 * QB) * 64) attn_fwd_wide_kernel
   }   // pass
 }
 
-template <typename T, int D, bool CAUSAL, int QB, int DBG = 0>
+// heads per group in the causal order "heaviest query blocks of a group's heads first" of the kernels that take one
+// 128-row query block per workgroup (see launch_one)
+static int heavy_first_group(const AttnParams& p, int D) {
+  const int64_t kv_bytes_head = (int64_t)p.Sk * D * 2 * 2, n_bh_x = ((int64_t)p.B * p.H) >> 3;
+  const int order = tune(g_attn_order);
+  int64_t group = order >= 0 ? order : 8 * n_bh_x * kv_bytes_head <= (256ll << 20) ? n_bh_x : (64ll << 20) / (8 * kv_bytes_head);
+  if (order < 0 && group < 1) group = 1;
+  if (group > n_bh_x) group = n_bh_x;
+  return (int)group;
+}
+
+// compute units of the current device (asked once per device; 256 where no device answers)
+static int device_cus() {
+  constexpr int kMaxDev = 64;
+  static std::atomic<int> cached[kMaxDev];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+template <typename T, int D, bool CAUSAL, int QB, int DBG = 0, int BM = kWideBM>
 static int launch_wide(AttnParams p, hipStream_t stream) {
   const size_t lds = 2 * (size_t)kRing * kBN * D * 2;
-  p.n_qblk = (p.Sq + kWideBM - 1) / kWideBM;
-  const unsigned grid = (unsigned)(wide_items(p.n_qblk, CAUSAL) * p.B * p.H);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG>,
+  p.n_qblk = (p.Sq + BM - 1) / BM;
+  const unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);
+  p.heavy_first = (CAUSAL && BM != kWideBM) ? heavy_first_group(p, D) : 0;
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
-  attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG><<<grid, kWideBM / (32 * QB) * 64, lds, stream>>>(p);
+  attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM><<<grid, BM / (32 * QB) * 64, lds, stream>>>(p);
   return launch_status();
 }
 
@@ -1119,12 +1164,7 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
   // (256 MiB) the heads are taken in groups whose K and V (over the eight XCDs) stay within a quarter of it - with
   // 512 heads of 1 MiB in one group the kernel is bound by HBM (0.90 ms against 0.67 ms).
   AttnParams q = p;
-  const int64_t kv_bytes_head = (int64_t)p.Sk * D * 2 * 2, n_bh_x = ((int64_t)p.B * p.H) >> 3;
-  const int order = tune(g_attn_order);
-  int64_t group = order >= 0 ? order : 8 * n_bh_x * kv_bytes_head <= (256ll << 20) ? n_bh_x : (64ll << 20) / (8 * kv_bytes_head);
-  if (order < 0 && group < 1) group = 1;
-  if (group > n_bh_x) group = n_bh_x;
-  q.heavy_first = CAUSAL ? (int)group : 0;
+  q.heavy_first = CAUSAL ? heavy_first_group(p, D) : 0;
   attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS><<<grid, kWaves * 64, lds, stream>>>(q);
   return launch_status();
 }
@@ -1140,7 +1180,7 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
   const bool wide_ok = (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
   // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
   // 128-row kernel, with four times as many workgroups, fills the chip better
-  static const int n_cu = [] { int dev = 0, n = 0; if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256; return n; }();
+  const int n_cu = device_cus();
   const int64_t wide_wgs = (int64_t)wide_items((p.Sq + kWideBM - 1) / kWideBM, causal) * p.B * p.H;
   int v = forced;
   if (forced < 0) {
@@ -1158,6 +1198,18 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // -0.5 %, 16384 -1.8 %; causal 2048 +10 %, 4096 +6.6 %, 6144 +5.5 %, 8192 +1.5 %, 16384 -1.2 %.
     if (D == 64 && keys < (causal ? 16384 : 8192)) wide = false;
     v = wide ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128;
+    // Few workgroups for the chip (12 heads of a tensor-parallel split, short batches): what bounds the launch then is
+    // the time a workgroup takes per key tile, not throughput, and 128-row workgroups in the pipelined kernel take less
+    // than the plain 128-row kernel (which runs S, the softmax and P V of a tile one after the other). Measured, plain
+    // against pipelined, head_dim 128 causal: 12 heads x 2048 45 -> 36 us, x 4096 87 -> 66 us, 32 heads x 2048 56 -> 50;
+    // non-causal 12 x 2048 46 -> 37, 8 x 4096 87 -> 72; head_dim 64 causal 12 x 4096 60 -> 50, 12 x 8192 139 -> 129. With
+    // more 128-row workgroups than the chip holds at once (twice that when causal, the average block being half) the
+    // other kernels are ahead again; below 1024 keys (2048 at head_dim 64) there is nothing to gain.
+    if (!wide && wide_ok) {
+      const int64_t wgs128 = ((int64_t)p.Sq + kBM - 1) / kBM * p.B * p.H;
+      const int64_t slots = (int64_t)n_cu * (D == 64 ? 2 : 1) * (causal ? 2 : 1);
+      if (wgs128 <= slots && keys >= (D == 64 ? 2048 : 1024)) v = FO_ATTN_KERNEL_ROWS128_PIPE;
+    }
     // head_dim 128 with many key tiles per query block: four waves x 64 rows. Every K / V^T fragment read from LDS feeds two
     // MFMAs, which costs less energy (at full load the chip's clock is what its power budget leaves) but more cycles per
     // tile, and its longer pipeline fill and drain have to be spread over enough tiles. Measured on one box, new form
@@ -1166,7 +1218,7 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     if (v == FO_ATTN_KERNEL_ROWS256_W8 && D == 128 && keys >= (causal ? 6144 : 2048)) v = FO_ATTN_KERNEL_ROWS256_W4;
   }
   if (v >= 256) return v;
-  if (!wide_ok && v >= 16) v = FO_ATTN_KERNEL_ROWS128;
+  if (!wide_ok && v >= FO_ATTN_KERNEL_ROWS128_PIPE) v = FO_ATTN_KERNEL_ROWS128;
   if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128) v = FO_ATTN_KERNEL_ROWS128;   // the four-wave form exists for head_dim 128 only
   return v;
 }
@@ -1180,6 +1232,7 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
   if (dropout) return causal ? launch_one<T, D, true, true, 0, true>(p, stream) : launch_one<T, D, false, true, 0, true>(p, stream);
   const int v = choose_kernel(p, D, causal, dropout, tune(g_attn_variant));
   if (v == FO_ATTN_KERNEL_ROWS256_W8) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
+  if (v == FO_ATTN_KERNEL_ROWS128_PIPE) return causal ? launch_wide<T, D, true, 1, 0, kBM>(p, stream) : launch_wide<T, D, false, 1, 0, kBM>(p, stream);
   if constexpr (D == 128) {
     if (v == FO_ATTN_KERNEL_ROWS256_W4) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
   }
@@ -1228,6 +1281,28 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
 
 using namespace fo;
 
+// The checks on sizes and strides that fo_attn_fwd and fo_attn_fwd_kernel share, so that the query answers "rejected"
+// exactly where the call would.
+static int check_sizes(int B, int H, int Sq, int Sk, int D) {
+  if (D < 8 || D > 128 || D % 8 != 0) return FO_ERR_BAD_HEAD_DIM;
+  if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return FO_ERR_BAD_SHAPE;
+  const int64_t n_qblk = ((int64_t)Sq + kBM - 1) / kBM;
+  if (n_qblk * B * H > 0x7FFFFFFFll || (int64_t)B * H * Sq > (1ll << 40)) return FO_ERR_BAD_SHAPE;
+  return FO_OK;
+}
+// three element strides (batch, head, sequence) of one operand: rows start on 16-byte boundaries (8 elements) and do not
+// overlap; only K/V may repeat a head (stride 0 = multi-query), which the caller checks for the output. The kernels
+// address the 64 rows of a key tile with 32-bit byte offsets (the 256-row kernel, whose offsets span a whole head, is
+// chosen only where they fit): a K/V row stride must stay below 2^24 elements.
+static int check_strides(const int64_t* st, int D, bool key_or_value) {
+  for (int i = 0; i < 3; ++i) {
+    if (st[i] < 0 || (st[i] % 8) != 0) return FO_ERR_BAD_STRIDE;
+  }
+  if (st[2] < D) return FO_ERR_BAD_STRIDE;
+  if (key_or_value && st[2] >= kMaxRowStride) return FO_ERR_BAD_STRIDE;
+  return FO_OK;
+}
+
 static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse,
                          int B, int H, int Sq, int Sk, int D,
                          const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
@@ -1235,23 +1310,14 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
                          const void* bias, const int64_t* bias_strides, int bias_dtype, void* stream) {
   if (!q || !k || !v || !o || !qs || !ks || !vs || !os) return FO_ERR_NULL_POINTER;
   if (dtype != FO_DTYPE_F16 && dtype != FO_DTYPE_BF16) return FO_ERR_BAD_DTYPE;
-  if (D < 8 || D > 128 || D % 8 != 0) return FO_ERR_BAD_HEAD_DIM;
-  if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return FO_ERR_BAD_SHAPE;
+  if (const int rc = check_sizes(B, H, Sq, Sk, D)) return rc;
   const int64_t n_qblk = ((int64_t)Sq + kBM - 1) / kBM;
-  if (n_qblk * B * H > 0x7FFFFFFFll || (int64_t)B * H * Sq > (1ll << 40)) return FO_ERR_BAD_SHAPE;
-  const int64_t* all[4] = {qs, ks, vs, os};
-  for (int t = 0; t < 4; ++t) {
-    // rows start on 16-byte boundaries (8 elements); only K/V may repeat a head (stride 0 = multi-query)
-    for (int i = 0; i < 3; ++i) {
-      if (all[t][i] < 0 || (all[t][i] % 8) != 0) return FO_ERR_BAD_STRIDE;
-    }
-    if (all[t][2] < D) return FO_ERR_BAD_STRIDE;
-  }
+  if (const int rc = check_strides(qs, D, false)) return rc;
+  if (const int rc = check_strides(ks, D, true)) return rc;
+  if (const int rc = check_strides(vs, D, true)) return rc;
+  if (const int rc = check_strides(os, D, false)) return rc;
   if (os[0] == 0 && B > 1) return FO_ERR_BAD_STRIDE;
   if (os[1] == 0 && H > 1) return FO_ERR_BAD_STRIDE;
-  // the 128-row kernel addresses the 64 rows of a key tile with 32-bit byte offsets (the 256-row kernel, whose offsets
-  // span a whole head, is chosen only where they fit): 63 * stride * 2 bytes must stay below 2^32
-  if (ks[2] >= kMaxRowStride || vs[2] >= kMaxRowStride) return FO_ERR_BAD_STRIDE;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15u) return FO_ERR_MISALIGNED;
   if (lse && ((uintptr_t)lse & 3u)) return FO_ERR_MISALIGNED;
   if (!(softmax_scale > 0.0f) || softmax_scale > 3.0e38f) return FO_ERR_BAD_SHAPE;   // also rejects NaN
@@ -1291,9 +1357,9 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
 extern "C" int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* ks, const int64_t* vs,
                                   int causal, int has_bias, int has_dropout) {
   if (!ks || !vs) return FO_ERR_NULL_POINTER;
-  if (D < 8 || D > 128 || D % 8 != 0) return FO_ERR_BAD_HEAD_DIM;
-  if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0) return FO_ERR_BAD_SHAPE;
-  if (ks[2] < D || vs[2] < D || ks[2] >= kMaxRowStride || vs[2] >= kMaxRowStride) return FO_ERR_BAD_STRIDE;
+  if (const int rc = check_sizes(B, H, Sq, Sk, D)) return rc;
+  if (const int rc = check_strides(ks, D, true)) return rc;
+  if (const int rc = check_strides(vs, D, true)) return rc;
   AttnParams p = {};
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.d = D;
   for (int i = 0; i < 3; ++i) { p.ks[i] = ks[i]; p.vs[i] = vs[i]; }

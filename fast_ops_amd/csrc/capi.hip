@@ -38,8 +38,9 @@ extern "C" int fo_tune_set(const char* key, int value) {
     fo::g_lion_variant = value; return FO_OK;
   }
   if (strcmp(key, "attn.variant") == 0) {
-    // FO_ATTN_KERNEL_*: 0 / 1 = 128-row kernel with the lazy / the exact rescale, 16 / 32 = 256-row kernel, 8 / 4 waves
-    bool ok = value == -1 || value == 0 || value == 1 || value == 16 || value == 32;
+    // FO_ATTN_KERNEL_*: 0 / 1 = 128-row kernel with the lazy / the exact rescale, 8 = 128 rows in the pipelined kernel,
+    // 16 / 32 = 256-row pipelined kernel with 8 / 4 waves
+    bool ok = value == -1 || value == 0 || value == 1 || value == 8 || value == 16 || value == 32;
 #if defined(FO_ABLATIONS)
     ok = true;
 #endif

@@ -92,6 +92,7 @@ int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
 enum {
   FO_ATTN_KERNEL_ROWS128 = 0,         /* 128 query rows per workgroup, reference maximum raised lazily */
   FO_ATTN_KERNEL_ROWS128_EXACT = 1,   /* the same with the exact running maximum of flash_attention_triton.py:200-213 */
+  FO_ATTN_KERNEL_ROWS128_PIPE = 8,    /* 128 query rows per workgroup, four waves x 32 rows, in the 256-row kernel's pipeline */
   FO_ATTN_KERNEL_ROWS256_W8 = 16,     /* 256 query rows per workgroup, eight waves x 32 rows */
   FO_ATTN_KERNEL_ROWS256_W4 = 32      /* 256 query rows per workgroup, four waves x 64 rows (head_dim 128 only) */
 };

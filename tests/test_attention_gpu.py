@@ -41,8 +41,9 @@ def _check(o, lse, o_ref, lse_ref, what=""):
 
 
 # attn.variant values: -1 = the library's choice (which depends on head_dim and on how many workgroups the shape gives),
+# 8 = 128 rows per workgroup in the pipelined kernel (four waves x 32 rows),
 # 0 = the 128-row kernel, 16 / 32 = the 256-row kernel with eight / four waves (four: head_dim 128 only)
-KERNELS_D128 = [-1, 0, 16, 32]
+KERNELS_D128 = [-1, 0, 8, 16, 32]
 
 
 @pytest.fixture
@@ -106,11 +107,21 @@ def test_dtype_causal_headdim_grid(dtype, causal, D):
     _run_and_check(2, 3, 512, 512, D, dtype, causal, seed=3)
 
 
-@pytest.mark.parametrize("kernel_variant", [0, 16, 32], indirect=True)
+@pytest.mark.parametrize("kernel_variant", [0, 8, 16, 32], indirect=True)
 def test_long_context_slice_of_headline_shape(kernel_variant):
     # the headline shape is B=2 H=16 S=8192 D=128 bf16 causal; two of its (batch, head) slices against the oracle, on each
     # of the three kernels (so few slices leave the choice to the 128-row kernel; the full shape is tested below)
     _run_and_check(1, 2, 8192, 8192, 128, torch.bfloat16, True, seed=0)
+
+
+@pytest.mark.parametrize("shape", [(1, 12, 2048, 128, True), (1, 12, 2048, 128, False), (1, 12, 4096, 64, True), (2, 6, 1024, 128, True)])
+def test_few_heads_take_the_128_row_pipelined_form(shape):
+    # the reference's own benchmark shapes, 12 heads per GPU (flash_attention/README.md:69-70): too few workgroups for the
+    # chip, so the library picks 128-row workgroups in the pipelined kernel; whole shape against the oracle
+    B, H, S, D, causal = shape
+    q, k, v = _qkv(B, H, S, S, D, torch.bfloat16, seed=S + D)
+    assert _kernel_taken(q, k, v, causal) == _lib.FO_ATTN_KERNEL_ROWS128_PIPE
+    _run_and_check(B, H, S, S, D, torch.bfloat16, causal, seed=S + D)
 
 
 def test_throughput_shape_slice_fp16_noncausal():
@@ -174,7 +185,7 @@ def test_headline_shape_on_both_forms_of_the_256_row_kernel(kernel_variant):
 @pytest.mark.parametrize("shape", [(1, 8, 1300, 1300), (2, 8, 800, 1000), (3, 8, 1111, 900), (1, 16, 1537, 1537)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
-@pytest.mark.parametrize("kernel_variant", [16, 32], indirect=True)
+@pytest.mark.parametrize("kernel_variant", [8, 16, 32], indirect=True)
 def test_256_row_kernel_with_heads_dealt_to_xcds_and_several_items_per_head(shape, causal, D, kernel_variant):
     # 8, 16 and 24 heads (a multiple of the 8 XCDs: workgroup id -> (XCD, head, item)) with 3 to 7 items per head, ragged
     # lengths; causal items are pairs of query blocks, the middle one single when their number is odd
@@ -211,7 +222,7 @@ def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype, kerne
 @pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
-@pytest.mark.parametrize("kernel_variant", [-1, 0, 16], indirect=True)
+@pytest.mark.parametrize("kernel_variant", [-1, 0, 8, 16], indirect=True)
 def test_ragged_across_256_row_blocks_head_dim_64(shape, causal, dtype, kernel_variant):
     B, H, Sq, Sk = shape
     _run_and_check(B, H, Sq, Sk, 64, dtype, causal, seed=Sq + Sk + 64)

@@ -161,9 +161,9 @@ def test_tune_hook_accepts_only_kernels_that_compute_the_function():
     # the shipped library holds no timing ablations (kernel variants that leave work out): their numbers select nothing
     lib = _lib.load()
     assert lib.fo_tune_get(b"build.ablations") == 0
-    for ok in (-1, 0, 1, 16, 32):
+    for ok in (-1, 0, 1, 8, 16, 32):
         assert lib.fo_tune_set(b"attn.variant", ok) == 0
-    for bad in (2, 3, 7, 8, 15, 17, 33, 257, 258, 260, 263, 320, 384, 519, 520, 640, -2):
+    for bad in (2, 3, 7, 9, 15, 17, 33, 257, 258, 260, 263, 320, 384, 519, 520, 640, -2):
         assert lib.fo_tune_set(b"attn.variant", bad) == -8, bad
         assert lib.fo_tune_get(b"attn.variant") == 32          # a refused value changes nothing
     assert lib.fo_tune_set(b"attn.variant", -1) == 0
@@ -191,8 +191,11 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     finally:
         lib.fo_tune_set(b"attn.variant", -1)
     assert k(1, 1, 128, 128, 76, 0) == -3 and k(0, 1, 128, 128, 64, 0) == -4
+    # the query refuses what the call refuses: sizes beyond the launch limits, strides that are negative or no multiple of 8
+    assert k(1 << 15, 1 << 15, 1 << 12, 128, 64, 0) == -4 and k(1 << 10, 1 << 10, 1 << 21, 128, 64, 0) == -4
+    assert k(1, 1, 128, 128, 64, 0, ks=I3(0, -8, 64)) == -5 and k(1, 1, 128, 128, 64, 0, ks=I3(0, 12, 64)) == -5
     # the library's own choice on 256 CUs (an MI355X, or what the library assumes where it finds no device)
-    R128, W8, W4 = _lib.FO_ATTN_KERNEL_ROWS128, _lib.FO_ATTN_KERNEL_ROWS256_W8, _lib.FO_ATTN_KERNEL_ROWS256_W4
+    R128, W8, W4, PIPE = _lib.FO_ATTN_KERNEL_ROWS128, _lib.FO_ATTN_KERNEL_ROWS256_W8, _lib.FO_ATTN_KERNEL_ROWS256_W4, _lib.FO_ATTN_KERNEL_ROWS128_PIPE
     assert k(2, 16, 8192, 8192, 128, 1) == W4            # the headline shape: 512 workgroups of two query blocks
     assert k(16, 32, 2048, 2048, 128, 0) == W4           # B=16 H=32 S=2048 non-causal
     assert k(8, 12, 1024, 1024, 64, 1) == R128           # the GPT-2-small shape
@@ -201,8 +204,13 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     assert k(12, 16, 1024, 1024, 128, 1) == R128         # 384 workgroups would leave half of the second round empty
     assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
     assert k(16, 16, 512, 512, 128, 0) == W8 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups
-    assert k(1, 8, 8192, 8192, 64, 0) == W8 and k(2, 8, 4096, 4096, 64, 0) == R128     # head_dim 64: long rows only
-    assert k(1, 8, 16384, 16384, 64, 1) == W8 and k(1, 16, 8192, 8192, 64, 1) == R128
+    assert k(1, 8, 8192, 8192, 64, 0) == W8 and k(4, 8, 4096, 4096, 64, 0) == R128     # head_dim 64: long rows only
+    assert k(1, 8, 16384, 16384, 64, 1) == W8 and k(2, 16, 8192, 8192, 64, 1) == R128
+    # too few workgroups for the chip (12 heads of a tensor-parallel split): 128-row workgroups in the pipelined kernel
+    assert k(1, 12, 2048, 2048, 128, 1) == PIPE and k(1, 12, 2048, 2048, 128, 0) == PIPE and k(1, 12, 4096, 4096, 128, 1) == PIPE
+    assert k(1, 12, 8192, 8192, 128, 1) == R128          # 768 workgroups of 128 rows: more than twice the chip
+    assert k(1, 12, 4096, 4096, 128, 0) == R128 and k(1, 12, 512, 512, 128, 0) == R128
+    assert k(1, 12, 4096, 4096, 64, 1) == PIPE and k(1, 12, 1024, 1024, 64, 1) == R128
     # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
     assert k(2, 16, 8192, 8192, 96, 1) == _lib.FO_ATTN_KERNEL_ROWS128
     assert lib.fo_attn_fwd_kernel(1, 1, 128, 128, 64, None, dense(128, 64), 0, 0, 0) == -1
