@@ -36,6 +36,8 @@ constexpr int kWaves = 4;
 constexpr int kBM = 32 * kWaves;   // query rows per workgroup
 constexpr int kBN = 64;            // keys per tile
 
+constexpr int kOrderTab = 128;
+
 struct AttnParams {
   const void* q; const void* k; const void* v; void* o; float* lse;
   int B, H, Sq, Sk;
@@ -44,6 +46,8 @@ struct AttnParams {
   float scale_log2e;                    // softmax_scale * log2(e)
   int n_qblk;
   int heavy_first;                      // 128-row kernel, causal: heads per group in the order of an XCD's workgroups, 0 = head by head (see launch_one)
+  int order_n;                          // 128-row kernel, causal: entries of order_tab in use, 0 = none
+  uint8_t order_tab[kOrderTab];         // position in an XCD's launch order -> rank of the workgroup (0 = heaviest) that runs there
   DropoutParams drop;                   // used by the kernels instantiated with dropout only
   BiasParams bias;                      // used by the kernels instantiated with bias only
 };
@@ -82,8 +86,10 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
       if (CAUSAL && prm.heavy_first > 0) {
         // groups of heavy_first heads; inside a group the heaviest query blocks of all its heads first
         const int n_bh_x = n_bh >> 3, per_group = prm.heavy_first * prm.n_qblk;
-        const int grp = j / per_group, r = j - grp * per_group;
+        const int grp = j / per_group;
+        int r = j - grp * per_group;
         const int heads = min(prm.heavy_first, n_bh_x - grp * prm.heavy_first);
+        if (prm.order_n > 0) r = prm.order_tab[r];      // (a launch whose workgroups are all resident at once: see launch_one)
         bh = x + 8 * (grp * prm.heavy_first + r % heads);
         qblk = prm.n_qblk - 1 - r / heads;
       } else {
@@ -1142,6 +1148,7 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
   p.n_qblk = (p.Sq + BM - 1) / BM;
   const unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);
   p.heavy_first = (CAUSAL && BM != kWideBM) ? heavy_first_group(p, D) : 0;
+  p.order_n = 0;
   static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
@@ -1165,6 +1172,34 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
   // 512 heads of 1 MiB in one group the kernel is bound by HBM (0.90 ms against 0.67 ms).
   AttnParams q = p;
   q.heavy_first = CAUSAL ? heavy_first_group(p, D) : 0;
+  q.order_n = 0;
+  if (CAUSAL && q.heavy_first > 0 && tune(g_attn_balance) != 0) {
+    // When an XCD's workgroups are all resident at once (three per compute unit at head_dim 64, two at 128), they are
+    // placed in launch order, one per unit in turn: unit m gets positions m, m + C, m + 2C of the XCD's list. In the
+    // plain heaviest-first order that is the m-th heaviest of every layer, and the units' sums differ widely
+    // (GPT-2-small shape, 96 workgroups per XCD on 32 units: 20 to 34 key tiles per unit). So the positions are filled
+    // from a table: workgroups by falling size, each to the unit with the least work so far that still has a position
+    // free (26 to 28 tiles per unit; 25.0 -> about 21 us). With more workgroups than fit at once the later ones start
+    // wherever a slot frees, and the plain order is the better one.
+    const int cus_x = device_cus() / 8, n_bh_x = (int)(((int64_t)p.B * p.H) >> 3);
+    const int64_t n = (int64_t)n_bh_x * p.n_qblk;
+    if (q.heavy_first == n_bh_x && cus_x > 0 && n <= (int64_t)cus_x * (D == 64 ? 3 : 2) && n <= kOrderTab && n > cus_x) {
+      int load[kOrderTab] = {0}, used[kOrderTab] = {0};
+      for (int rank = 0; rank < (int)n; ++rank) {
+        const int qblk = p.n_qblk - 1 - rank / n_bh_x;
+        const int tiles = ((p.Sk < (qblk + 1) * kBM ? p.Sk : (qblk + 1) * kBM) + kBN - 1) / kBN;
+        int best = -1;
+        for (int m = 0; m < cus_x; ++m) {
+          const int cap = (int)((n - m + cus_x - 1) / cus_x);      // positions m, m + C, ... below n
+          if (used[m] < cap && (best < 0 || load[m] < load[best])) best = m;
+        }
+        q.order_tab[used[best] * cus_x + best] = (uint8_t)rank;
+        load[best] += tiles;
+        used[best] += 1;
+      }
+      q.order_n = (int)n;
+    }
+  }
   attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS><<<grid, kWaves * 64, lds, stream>>>(q);
   return launch_status();
 }
@@ -1189,7 +1224,11 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // With the rounds filled to less than 80 % the 128-row kernel (two workgroups per CU, finer blocks, heaviest first)
     // was 1-5 % faster (B*H = 160-192 at 512-1024 keys, 48 heads x 4096 causal), from 83 % on the 256-row kernel 3-6 %.
     const int64_t rounds = (wide_wgs + n_cu - 1) / n_cu;
-    bool wide = wide_ok && wide_wgs >= n_cu && wide_wgs * 5 >= rounds * n_cu * 4;
+    bool wide = wide_ok && wide_wgs >= n_cu && wide_wgs * 10 >= rounds * n_cu * (D == 128 && keys >= 4096 ? 7 : 8);
+    // (long rows of keys at head_dim 128: also with the rounds filled to 70-80 % - 12 heads x 8192 non-causal, 384
+    // workgroups, 375 against 399 us - and with three quarters of a single round - 12 heads x 8192 causal 196 against 215 us,
+    // 12 heads x 4096 non-causal 98 against 121 us)
+    if (wide_ok && D == 128 && keys >= 4096 && wide_wgs < n_cu && wide_wgs * 4 >= (int64_t)n_cu * 3) wide = true;
     // head_dim 128, causal: from 1024 queries on (B*H = 128: 1024 queries -8 %, 1536 -16 %, 2048 -12 % against the
     // 128-row kernel; 512 and 768 queries +7 % and +18 %, a 256-row block being a large part of so small a triangle).
     if (D == 128 && causal && p.Sq < 1024) wide = false;

@@ -32,7 +32,7 @@ def _half_precision_torch(q, k, v, go, causal, scale):
     s = (qa * scale) @ ka.transpose(-1, -2)
     if causal:
         M, N = q.shape[2], k.shape[2]
-        s = s.masked_fill(torch.arange(N)[None, :] > torch.arange(M)[:, None], float("-inf"))
+        s = s.masked_fill(torch.arange(N, device=q.device)[None, :] > torch.arange(M, device=q.device)[:, None], float("-inf"))
     o = torch.softmax(s.float(), dim=-1).to(q.dtype) @ va
     return torch.autograd.grad(o, (qa, ka, va), go)
 
@@ -114,7 +114,9 @@ def test_long_context_slice_of_headline_shape(causal, dkdv_variant):
 def test_headline_shape_whole_with_the_benchmarks_dispatch():
     # B=2 H=16 S=8192 D=128 bf16 causal as bench.py runs it: 32 heads dealt to the 8 XCDs, 64 key blocks and 64 query
     # blocks per head, the library's own choice of kernels and workgroup order. Six (batch, head) slices that lie on six
-    # different XCDs, first and last head included, against the fp32 closed form (absolute criterion as above).
+    # different XCDs, first and last head included, against the fp32 closed form: the first and the last slice by the
+    # reference's criterion (tests/test_flash_attention_triton.py:137-141: at most twice the error of the same expression in
+    # the operand dtype, which is run on the GPU here as the reference runs it), the others by the absolute criterion.
     B, H, S, D = 2, 16, 8192, 128
     q, k, v, go = _inputs(B, H, S, S, D, torch.bfloat16, seed=4)
     qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
@@ -125,6 +127,10 @@ def test_headline_shape_whole_with_the_benchmarks_dispatch():
     for b, h in slices:
         sl = (slice(b, b + 1), slice(h, h + 1))
         ref = attention_bwd_oracle(q[sl], k[sl], v[sl], go[sl], causal=True)
+        if (b, h) in ((0, 0), (1, 15)):
+            pt = [t.cpu() for t in _half_precision_torch(q[sl].to(DEV), k[sl].to(DEV), v[sl].to(DEV), go[sl].to(DEV), True, 1.0 / math.sqrt(D))]
+            _check([a[sl] for a in got], ref, pt, f"headline shape, slice ({b},{h})")
+            continue
         for name, a, r in zip(("dQ", "dK", "dV"), got, ref):
             e = (a[sl].float() - r).abs().max().item()
             assert math.isfinite(e) and e <= 2e-2 * max(1.0, r.abs().max().item()), f"slice ({b},{h}) {name}: error {e:.3e} vs magnitude {r.abs().max().item():.3e}"

@@ -87,9 +87,9 @@ def test_config2_gpt2_small_bf16_causal():
 @pytest.mark.parametrize("heads", [(2, 4), (5, 8), (3, 5)])
 def test_causal_workgroup_order_of_128_row_kernel(group, heads):
     # attn.order: how many of an XCD's heads form a group whose heaviest query blocks run first (0: head by head, -1:
-    # the library's choice). Every (head, query block) must be computed exactly once whatever the grouping, also when
-    # the last group is smaller than the others (40 heads = 5 per XCD in groups of 2 or 3) and when the number of heads
-    # is no multiple of the 8 XCDs (15 heads: the grouping does not apply).
+    # the library's choice). Every (head, query block) must be computed exactly once whatever the grouping, also when the
+    # last group is smaller than the others (40 heads = 5 per XCD in groups of 2 or 3) and when the number of heads is no
+    # multiple of the 8 XCDs (15 heads: the grouping does not apply).
     B, H = heads
     _lib.tune_set("attn.variant", 0)
     _lib.tune_set("attn.order", group)
@@ -98,6 +98,22 @@ def test_causal_workgroup_order_of_128_row_kernel(group, heads):
     finally:
         _lib.tune_set("attn.variant", -1)
         _lib.tune_set("attn.order", -1)
+
+
+@pytest.mark.parametrize("balance", [-1, 0])
+@pytest.mark.parametrize("shape", [(8, 12, 1024, 64), (4, 16, 1024, 64), (5, 8, 700, 64), (2, 20, 1100, 64), (8, 5, 1536, 128), (3, 8, 900, 128), (8, 9, 1024, 64)])
+def test_balanced_order_of_a_launch_that_fits_the_chip_at_once(shape, balance):
+    # attn.balance: a causal launch of the 128-row kernel whose workgroups are all resident at once takes its order from a
+    # table (heaviest first, each to the compute unit with the least work so far) - whole shapes against the oracle, with
+    # the table (33 to 96 workgroups per XCD: full and ragged last layers, two and three layers) and without it
+    B, H, S, D = shape
+    _lib.tune_set("attn.variant", 0)
+    _lib.tune_set("attn.balance", balance)
+    try:
+        _run_and_check(B, H, S, S, D, torch.bfloat16, True, seed=S + H)
+    finally:
+        _lib.tune_set("attn.variant", -1)
+        _lib.tune_set("attn.balance", -1)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)

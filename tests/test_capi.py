@@ -151,7 +151,7 @@ def test_tune_hook():
     assert lib.fo_tune_set(b"lion.variant", -1) == 0
     assert lib.fo_tune_set(b"no.such.key", 1) == -8
     # every key the kernels read: default -1 (the library's choice), settable, readable
-    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn_bwd.order", 2)):
+    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn.balance", 0), (b"attn_bwd.order", 2)):
         assert lib.fo_tune_get(key) == -1
         assert lib.fo_tune_set(key, value) == 0 and lib.fo_tune_get(key) == value
         assert lib.fo_tune_set(key, -1) == 0 and lib.fo_tune_get(key) == -1
@@ -208,8 +208,9 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     assert k(1, 8, 16384, 16384, 64, 1) == W8 and k(2, 16, 8192, 8192, 64, 1) == R128
     # too few workgroups for the chip (12 heads of a tensor-parallel split): 128-row workgroups in the pipelined kernel
     assert k(1, 12, 2048, 2048, 128, 1) == PIPE and k(1, 12, 2048, 2048, 128, 0) == PIPE and k(1, 12, 4096, 4096, 128, 1) == PIPE
-    assert k(1, 12, 8192, 8192, 128, 1) == R128          # 768 workgroups of 128 rows: more than twice the chip
-    assert k(1, 12, 4096, 4096, 128, 0) == R128 and k(1, 12, 512, 512, 128, 0) == R128
+    # long rows of keys at head_dim 128: the 256-row kernel already with three quarters of one round of workgroups
+    assert k(1, 12, 8192, 8192, 128, 1) == W4 and k(1, 12, 4096, 4096, 128, 0) == W4 and k(1, 12, 8192, 8192, 128, 0) == W4
+    assert k(1, 10, 8192, 8192, 128, 1) == R128 and k(1, 12, 512, 512, 128, 0) == R128
     assert k(1, 12, 4096, 4096, 64, 1) == PIPE and k(1, 12, 1024, 1024, 64, 1) == R128
     # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
     assert k(2, 16, 8192, 8192, 96, 1) == _lib.FO_ATTN_KERNEL_ROWS128
