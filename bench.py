@@ -139,7 +139,7 @@ def _attn_inputs(B, H, S, D, dtype, dev, seed=0):
     return tuple(torch.randn(B, H, S, D, generator=g).to(dtype).to(dev) for _ in range(3)), g
 
 
-KERNEL_NAMES = {0: "rows128", 1: "rows128_exact", 16: "rows256_w8", 32: "rows256_w4"}
+KERNEL_NAMES = {0: "rows128", 1: "rows128_exact", 8: "rows128_pipelined", 16: "rows256_w8", 32: "rows256_w4"}
 
 
 def _attn_rate(B, H, S, D, dtype, causal, steps, warmup, settle, operands="normal", backward=False):
@@ -173,7 +173,8 @@ def _attn_rate(B, H, S, D, dtype, causal, steps, warmup, settle, operands="norma
                     + (", all-zero operands" if operands == "zero" else ""),
         "ms_per_step": ms_step, "kernel_ms_avg": ms_kernel, "kernel_ms_min": ms_min, "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "achieved": flops / (ms_kernel * 1e-3) / 1e12, "frac": flops / (ms_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": flops,
-        "kernel": KERNEL_NAMES.get(kernel, str(kernel)), "kernel_ms_median": info["kernel_ms_median"], "settle": info,
+        "kernel": KERNEL_NAMES.get(kernel, str(kernel)), "kernel_ms_median": info["kernel_ms_median"],
+        "frac_median": flops / (info["kernel_ms_median"] * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "settle": info,
     }
     if backward:
         go = torch.randn(B, H, S, D, generator=g).to(dtype).to("cuda:0")
@@ -182,7 +183,8 @@ def _attn_rate(B, H, S, D, dtype, causal, steps, warmup, settle, operands="norma
         b_step, b_kernel, b_min, b_info = _time_steps(lambda: attn_bwd_strided(q, k, v, o_fix, lse_fix, go, (0, 1, 2, 3), causal, scale),
                                                       steps, warmup, settle // 2, wall_without_events=True)
         res["bwd"] = {"ms_per_step": b_step, "kernel_ms_avg": b_kernel, "kernel_ms_min": b_min, "kernel_ms_median": b_info["kernel_ms_median"], "value": bflops / (b_step * 1e-3) / 1e12, "unit": "TFLOP/s",
-                      "frac": bflops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": bflops,
+                      "frac": bflops / (b_kernel * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS,
+                      "frac_median": bflops / (b_info["kernel_ms_median"] * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, "flops_per_launch": bflops,
                       "what": "dQ + dK/dV launches of the same shape, FLOPs by the five-GEMM count"}
     return res
 

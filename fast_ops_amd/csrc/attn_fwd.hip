@@ -1183,20 +1183,29 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
     // wherever a slot frees, and the plain order is the better one.
     const int cus_x = device_cus() / 8, n_bh_x = (int)(((int64_t)p.B * p.H) >> 3);
     const int64_t n = (int64_t)n_bh_x * p.n_qblk;
-    if (q.heavy_first == n_bh_x && cus_x > 0 && n <= (int64_t)cus_x * (D == 64 ? 3 : 2) && n <= kOrderTab && n > cus_x) {
-      int load[kOrderTab] = {0}, used[kOrderTab] = {0};
-      for (int rank = 0; rank < (int)n; ++rank) {
-        const int qblk = p.n_qblk - 1 - rank / n_bh_x;
-        const int tiles = ((p.Sk < (qblk + 1) * kBM ? p.Sk : (qblk + 1) * kBM) + kBN - 1) / kBN;
-        int best = -1;
-        for (int m = 0; m < cus_x; ++m) {
-          const int cap = (int)((n - m + cus_x - 1) / cus_x);      // positions m, m + C, ... below n
-          if (used[m] < cap && (best < 0 || load[m] < load[best])) best = m;
+    const int resident = (D == 64 && !DROP && !BIAS) ? 3 : 2;      // workgroups per compute unit (registers)
+    if (q.heavy_first == n_bh_x && cus_x > 0 && cus_x <= kOrderTab && n <= (int64_t)cus_x * resident && n <= kOrderTab && n > cus_x) {
+      // (the table of the last shape is kept per host thread: filling it takes a few microseconds, a training loop
+      // launches the same shape over and over)
+      struct Memo { int n, n_bh_x, n_qblk, Sk, cus_x; uint8_t tab[kOrderTab]; };
+      static thread_local Memo memo = {0, 0, 0, 0, 0, {0}};
+      if (memo.n != (int)n || memo.n_bh_x != n_bh_x || memo.n_qblk != p.n_qblk || memo.Sk != p.Sk || memo.cus_x != cus_x) {
+        int load[kOrderTab] = {0}, used[kOrderTab] = {0};
+        for (int rank = 0; rank < (int)n; ++rank) {
+          const int qblk = p.n_qblk - 1 - rank / n_bh_x;
+          const int tiles = ((p.Sk < (qblk + 1) * kBM ? p.Sk : (qblk + 1) * kBM) + kBN - 1) / kBN;
+          int best = -1;
+          for (int m = 0; m < cus_x; ++m) {
+            const int cap = (int)((n - m + cus_x - 1) / cus_x);      // positions m, m + C, ... below n
+            if (used[m] < cap && (best < 0 || load[m] < load[best])) best = m;
+          }
+          memo.tab[used[best] * cus_x + best] = (uint8_t)rank;
+          load[best] += tiles;
+          used[best] += 1;
         }
-        q.order_tab[used[best] * cus_x + best] = (uint8_t)rank;
-        load[best] += tiles;
-        used[best] += 1;
+        memo.n = (int)n; memo.n_bh_x = n_bh_x; memo.n_qblk = p.n_qblk; memo.Sk = p.Sk; memo.cus_x = cus_x;
       }
+      for (int i = 0; i < (int)n; ++i) q.order_tab[i] = memo.tab[i];
       q.order_n = (int)n;
     }
   }
