@@ -48,7 +48,7 @@ SOURCES = {
 # sources whose generated assembly is checked by asm_lint: source -> regular expression of the kernel symbols to check
 # (the instantiations with a non-zero last template argument are timing experiments with wrong results by design)
 # (attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM>: DBG is the last but one)
-ASM_LINTED = {"attn_fwd.hip": r"attn_fwd_wide_kernel.*ELi0ELi\d+EEEvNS_10AttnParamsE", "attn_bwd.hip": r"attn_bwd_dkdv_pipe_kernel"}
+ASM_LINTED = {"attn_fwd.hip": r"attn_fwd_wide_kernel.*ELi0ELi\d+ELb[01]EEEvNS_10AttnParamsE", "attn_bwd.hip": r"attn_bwd_dkdv_pipe_kernel"}
 
 
 def _hipcc() -> str:

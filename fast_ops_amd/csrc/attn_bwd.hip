@@ -216,8 +216,15 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
 constexpr int stage_bytes(int D) { return 32 * (D * 2 + 16); }   // per wave and matrix
 
 // ---------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS>
+// KBIAS (without BIAS): a bias that is the same for every query (query stride 0), at no cost per score. Its 64
+// values of a key tile, divided by softmax_scale, are what the accumulators of S^T start from - register r of a lane
+// holds a key that depends on r and the half of the wave only - so that the MFMAs deliver S + b / scale and everything
+// after them is the code without bias. Wave 0 fetches the values of tile t+2 while tile t is worked on (a plain load: it
+// is waited for at the top of the next tile, where every copy in flight is waited for anyway), converts those of tile
+// t+1 and puts them into LDS, where every wave reads them after the next barrier.
+template <typename T, int D, bool CAUSAL, bool DROP, bool BIAS, bool KBIAS = false>
 __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const AttnBwdParams prm) {
+  static_assert(!(KBIAS && BIAS), "one bias form at a time");
   typedef typename Ops<T>::vec8 vec8;
   constexpr int TILE_BYTES = kBwdTile * D * 2;
   constexpr int KSTEPS = D / 16;
@@ -270,6 +277,16 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     }
   };
   issue(0, 0);
+  FO_LDS float* key_bias = (FO_LDS float*)(smem + 4 * TILE_BYTES);      // KBIAS: [2][64], bias / scale of the keys of a tile
+  float key_bias_next = 0.0f;                                           // (wave 0) this lane's key of the tile after next
+  const float per_scale = KBIAS ? kLog2e / prm.scale_log2e : 0.0f;
+  const int64_t key_bias_row = KBIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] : 0;
+  if constexpr (KBIAS) {
+    if (wave_s == 0) {
+      key_bias[lane] = load_bias<T>(prm.bias, key_bias_row + min(lane, Sk - 1)) * per_scale;
+      key_bias_next = load_bias<T>(prm.bias, key_bias_row + min(kBwdTile + lane, Sk - 1));
+    }
+  }
 
   // B operands held for the whole kernel: Q^T and dO^T fragments of this lane's query row; its LSE and delta
   const int qrow = min(q0w + l32, Sq - 1);
@@ -317,7 +334,18 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     const int key0 = tile * kBwdTile;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if constexpr (KBIAS) {
+      // (the value fetched one tile ago is used before this tile's copies go out: the wait the compiler puts in front
+      // of its use then finds nothing in flight)
+      if (wave_s == 0) {
+        asm volatile("" : "+v"(key_bias_next));                                  // (the use starts here, not earlier)
+        key_bias[(buf ^ 1) * kBwdTile + lane] = key_bias_next * per_scale;       // tile + 1: read after the next barrier
+      }
+    }
     if (tile + 1 < n_tiles) issue(tile + 1, buf ^ 1);
+    if constexpr (KBIAS) {
+      if (wave_s == 0) key_bias_next = load_bias<T>(prm.bias, key_bias_row + min((tile + 2) * kBwdTile + lane, Sk - 1));
+    }
     if (CAUSAL && key0 > q0w + 31) continue;
     FO_LDS const char* kt = smem + buf * TILE_BYTES;
     FO_LDS const char* vt = smem + (2 + buf) * TILE_BYTES;
@@ -327,6 +355,16 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sacc[kb][r] = 0.0f; dpacc[kb][r] = 0.0f; }
+    if constexpr (KBIAS) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int jv = 0; jv < 4; ++jv) {
+          const f32x4 b4 = *(FO_LDS const f32x4*)(key_bias + buf * kBwdTile + 32 * kb + 8 * jv + 4 * hh);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) sacc[kb][4 * jv + u] = b4[u];
+        }
+    }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
@@ -720,7 +758,9 @@ static_assert(softmax_grad_jobs_fit(16) && softmax_grad_jobs_fit(8), "head_dim 1
 // S and dP do not start from zero but from -LSE / scale and -delta of their rows (written by the dQ kernel, read from
 // LDS straight into the registers while they are idle), so that P = exp2((QK^T - LSE / scale) c) and dS = P (dP - delta)
 // are two multiplications and the exponential.
-template <typename T, int D, bool CAUSAL>
+// KBIAS: with a bias that is the same for every query (query stride 0): a lane owns a key, so the bias is one value per
+// lane for the whole kernel, and P = exp2(S c + b log2 e) is a fused multiply-add where the form without bias multiplies.
+template <typename T, int D, bool CAUSAL, bool KBIAS = false>
 __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(const AttnBwdParams prm) {
   typedef typename Ops<T>::vec8 vec8;
   constexpr int TILE_BYTES = kBwdTile * D * 2;
@@ -798,6 +838,11 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
     for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(kf[ks]), "v"(vf[ks]));
   }
   const int key = k0w + l32;
+  float bias_lane = 0.0f;
+  if constexpr (KBIAS) {
+    bias_lane = load_bias<T>(prm.bias, b * prm.bias.strides[0] + h * prm.bias.strides[1] + min(key, Sk - 1)) * kLog2e;
+    asm volatile("" : "+v"(bias_lane));      // (waited for here, not inside the loops, where copies are in flight)
+  }
   f32x16 dkacc[DBLK], dvacc[DBLK];
 #pragma unroll
   for (int i = 0; i < DBLK; ++i)
@@ -907,7 +952,7 @@ __global__ void __launch_bounds__(kBwdWaves * 64) attn_bwd_dkdv_pipe_kernel(cons
         const int lim_end = Sq - (q0t + 32 * qb + 4 * hh);
         dead = koff < lim || koff >= lim_end;
       }
-      pv[qb][r] = dead ? 0.0f : __builtin_amdgcn_exp2f(sacc[qb][r] * c);
+      pv[qb][r] = dead ? 0.0f : __builtin_amdgcn_exp2f(KBIAS ? __builtin_fmaf(sacc[qb][r], c, bias_lane) : sacc[qb][r] * c);
     };
     auto stage_b = [&](int qb, int r) {          // elements r and r + 1
       const float ds0 = pv[qb][r] * dpacc[qb][r], ds1 = pv[qb][r + 1] * dpacc[qb][r + 1];
@@ -1055,7 +1100,7 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   const int64_t g_dkdv = ((p.Sk + kBwdRows - 1) / kBwdRows) * n_bh;
   if (g_dq > 0x7FFFFFFFll || g_dkdv > 0x7FFFFFFFll) return FO_ERR_BAD_SHAPE;
   const size_t lds_tiles = 4 * (size_t)kBwdTile * D * 2;
-  const size_t lds_dq = lds_tiles + (BIAS ? 512 : 0);   // + the per-key bias of two tiles
+  const size_t lds_dq = lds_tiles + (BIAS ? 512 : 0);   // + the per-key bias of two tiles (both bias forms)
   const size_t lds_dkdv = lds_tiles + 4 * kBwdTile * sizeof(float) + (BIAS ? kBwdWaves * 2 * kBwdTile * 32 * 4 : 0);   // + bias tiles
   static const hipError_t a1 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
@@ -1065,6 +1110,16 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   static const hipError_t a3 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pipe);
   if (a1 != hipSuccess || a2 != hipSuccess || a3 != hipSuccess) return FO_ERR_LAUNCH;
+  // a bias without a query stride: the forms of the dQ kernel and (without dropout) of the pipelined dK/dV kernel that
+  // take it at no cost per score (attn_bwd.variant 0 keeps the general bias kernels, which tests compare them with)
+  const bool key_bias = BIAS && p.bias.strides[2] == 0 && tune(g_attn_bwd_variant) != 0;
+  if constexpr (BIAS) {
+    static const hipError_t a4 = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<T, D, CAUSAL, DROP, false, true>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
+    static const hipError_t a5 = hipFuncSetAttribute((const void*)attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL, true>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pipe);
+    if (a4 != hipSuccess || a5 != hipSuccess) return FO_ERR_LAUNCH;
+  }
   // one group while the Q, dO, K and V of all heads fit the memory-side cache (256 MiB), else groups of heads whose
   // operands stay within a quarter of it; multiples of 8 so that a head's workgroups keep landing on one XCD
   // (B=16 H=32 S=2048 D=128 causal: 2.61 ms in one group, 2.23 ms in groups of 32; the headline shape, 256 MiB: 1.80 ms
@@ -1079,6 +1134,14 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
     q.head_group = (int)group;
   }
   // (delta is computed by the dQ kernel, which the dK/dV kernel follows)
+  if constexpr (BIAS) {
+    if (key_bias) {
+      attn_bwd_dq_kernel<T, D, CAUSAL, DROP, false, true><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(q);
+      if (!DROP && p.d == D) attn_bwd_dkdv_pipe_kernel<T, D, CAUSAL, true><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_pipe, s>>>(q);
+      else attn_bwd_dkdv_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dkdv, kBwdWaves * 64, lds_dkdv, s>>>(q);
+      return launch_status();
+    }
+  }
   attn_bwd_dq_kernel<T, D, CAUSAL, DROP, BIAS><<<(unsigned)g_dq, kBwdWaves * 64, lds_dq, s>>>(q);
   // attn_bwd.variant 0 selects the plain dK/dV kernel everywhere (tests compare the two)
   // (and every head_dim other than the two the kernels are compiled for)

@@ -55,8 +55,14 @@ struct AttnParams {
 constexpr int64_t kMaxRowStride = 1ll << 24;   // elements; see attn_fwd_impl
 constexpr float kLazyLog2 = 8.0f;   // how far (in log2 units) a tile maximum may exceed the reference before a rescale
 
-template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false>
+// KBIAS (without BIAS): a bias that is the same for every query (query stride 0) at no cost per score. The 64 values of a
+// key tile, divided by softmax_scale, are what the score accumulators start from (register r of a lane holds a key that
+// depends on r and the half of the wave only), so the MFMAs deliver S + b / scale and the rest is the code without bias.
+// Wave 0 fetches the values of tile t+2 while tile t is worked on (a plain load, waited for at the top of the next tile,
+// where every copy in flight is waited for anyway), converts those of tile t+1 and puts them into LDS for everyone.
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false, bool KBIAS = false>
 __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnParams prm) {
+  static_assert(!(KBIAS && BIAS), "one bias form at a time");
   typedef typename Ops<T>::vec8 vec8;
   constexpr int ROW_BYTES = D * 2;
   constexpr int CHUNKS = ROW_BYTES / 16;            // 16-byte chunks per row
@@ -196,6 +202,16 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
 
   issue_tile(0, 0);
   if constexpr (BIAS) issue_bias(0, 0);
+  FO_LDS float* key_bias = (FO_LDS float*)(smem + 4 * TILE_BYTES);      // KBIAS: [2][64], bias / scale of the keys of a tile
+  float key_bias_next = 0.0f;                                           // (wave 0) this lane's key of the tile after next
+  const float per_scale = KBIAS ? 1.4426950408889634f / prm.scale_log2e : 0.0f;
+  const int64_t key_bias_row = KBIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] : 0;
+  if constexpr (KBIAS) {
+    if (wave_s == 0) {
+      key_bias[lane] = load_bias<T>(prm.bias, key_bias_row + min(lane, Sk - 1)) * per_scale;
+      key_bias_next = load_bias<T>(prm.bias, key_bias_row + min(kBN + lane, Sk - 1));
+    }
+  }
 
   // ---- Q^T fragments (B operand): lane holds query row q0w + l32, d = 16*ks + 8*hh .. +7
   vec8 qf[KSTEPS];
@@ -232,8 +248,19 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const int key0 = tile * kBN;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's pieces of tile `tile` have landed in LDS
     if (!(DBG & 4)) __syncthreads();        // everyone's pieces have landed; everyone is done reading the other buffer
+    if constexpr (KBIAS) {
+      // (the value fetched one tile ago is used before this tile's copies go out: the wait the compiler puts in front
+      // of its use then finds nothing in flight)
+      if (wave_s == 0) {
+        asm volatile("" : "+v"(key_bias_next));
+        key_bias[(buf ^ 1) * kBN + lane] = key_bias_next * per_scale;   // tile + 1: read after the next barrier
+      }
+    }
     if (tile + 1 < n_tiles && (!(DBG & 1) || tile < 1)) issue_tile(tile + 1, buf ^ 1);
     if constexpr (BIAS) { if (tile + 1 < n_tiles) issue_bias(tile + 1, buf ^ 1); }
+    if constexpr (KBIAS) {
+      if (wave_s == 0) key_bias_next = load_bias<T>(prm.bias, key_bias_row + min((tile + 2) * kBN + lane, Sk - 1));
+    }
 
     // waves whose rows are all above this tile's keys have nothing to do (causal)
     if (CAUSAL && key0 > q0w + 31) continue;
@@ -261,6 +288,16 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.0f;
+      if constexpr (KBIAS) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int jv = 0; jv < 4; ++jv) {
+            const f32x4 b4 = *(FO_LDS const f32x4*)(key_bias + buf * kBN + 32 * kb + 8 * jv + 4 * hh);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sacc[kb][4 * jv + u] = b4[u];
+          }
+      }
       vec8 fa[GK], fb[GK];
       load_group(0, fa);
 #pragma unroll
@@ -366,7 +403,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
     const bool raise = LAZY ? (mloc * c > m_run * c + kLazyLog2) : (mloc > m_run);
     if (__builtin_amdgcn_ballot_w64(raise) != 0) {
       const float m_new = fmaxf(m_run, mloc);          // finite from the first tile on: key 0 is never masked
-      const float alpha = (BIAS && m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      const float alpha = ((BIAS || KBIAS) && m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c);
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -375,7 +412,7 @@ __global__ void __launch_bounds__(kWaves * 64, 2) attn_fwd_kernel(const AttnPara
         for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
     }
     // a bias may mask every key seen so far (-inf, e.g. left padding): the reference then stays 0 until a key counts
-    const float mc = (BIAS && m_run == -INFINITY) ? 0.0f : m_run * c;
+    const float mc = ((BIAS || KBIAS) && m_run == -INFINITY) ? 0.0f : m_run * c;
     float psum = 0.0f;
     vec8 pf[4];
     // dropout: 32-bit index of this lane's query row at key 0 of the tile (flash_attention_triton.py:125,217)
@@ -565,8 +602,19 @@ __device__ __forceinline__ void scale_acc(f32x16& acc, float a) {
 // workgroups per head of the wide kernel
 __host__ __device__ inline int wide_items(int n_qblk, bool causal) { return causal ? (n_qblk + 1) / 2 : n_qblk; }
 
-template <typename T, int D, bool CAUSAL, int QB, int DBG, int BM = kWideBM>
-__global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 128) ? 1 : 2) attn_fwd_wide_kernel(const AttnParams prm) {
+// keys of a per-key bias the pipelined kernel keeps in LDS (fp32, beside the rings: 128 + 32 of the 160 KiB at head_dim 128)
+constexpr int kVBiasKeys = 8192;
+
+template <typename T, int D, bool CAUSAL, int QB, int DBG, int BM = kWideBM, bool VBIAS = false>
+__global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 128 || VBIAS) ? 1 : 2) attn_fwd_wide_kernel(const AttnParams prm) {
+  // VBIAS: an additive bias that is the same for every query of a head (query stride 0: the reference's "vector" bias,
+  // flash_attention_triton.py:176-186, e.g. a key padding mask). The head's row of it, at most kVBiasKeys keys, is put
+  // into LDS once per workgroup as fp32 divided by softmax_scale, so that (S + b / scale) * scale * log2 e is the biased
+  // score in the base-2 domain and the running maximum, the lazily raised reference and LSE keep their meaning with
+  // S + b / scale in the place of S. A step reads the 16 values of its 32 keys that a lane's registers hold (they
+  // depend on the register and the half of the wave only) and adds them where the scores are scaled: one more VALU
+  // instruction per score. A bias of -inf removes a key; rows whose keys so far are all removed have the reference
+  // -inf, and every step of such a row takes the recovery path (left padding: a few steps per workgroup).
   // BM = 256: the form described above. BM = 128 (QB = 1): the same pipeline with four waves x 32 rows, one query block
   // per workgroup in the 128-row kernel's order (heaviest causal blocks first), for shapes that give the chip too few
   // 256-row workgroups: a workgroup's time per key tile is what bounds those, and this pipeline's is less than half the
@@ -642,6 +690,15 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
       for (int ks = 0; ks < KSTEPS; ++ks) qf[qb][ks] = *(const i32x4*)(qp + 16 * ks);
     }
   };
+  FO_LDS float* vbias = (FO_LDS float*)(smem + 2 * kRing * TILE_BYTES) + 4 * hh;   // (this lane's half: its registers' keys start 4 further)
+  if constexpr (VBIAS) {
+    const int64_t brow = b * prm.bias.strides[0] + h * prm.bias.strides[1];
+    const float per_scale = 1.4426950408889634f / prm.scale_log2e;
+    const int n_pad = (prm.Sk + kBN - 1) / kBN * kBN;                  // at most kVBiasKeys: the launcher checks
+    for (int i = tid; i < n_pad; i += kWideWaves * 64)
+      ((FO_LDS float*)(smem + 2 * kRing * TILE_BYTES))[i] = load_bias<T>(prm.bias, brow + min(i, prm.Sk - 1)) * per_scale;
+    __syncthreads();
+  }
   for (int pass = 0; pass < n_pass; ++pass) {
   const int qblk = PAIRED ? (pass == 0 ? prm.n_qblk - 1 - item : item) : item;
   if (pass > 0) {
@@ -845,6 +902,7 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
       dma_dst = smem + ((P == 0 ? 0 : kRing) + (dma_tile & (kRing - 1))) * TILE_BYTES + wave_s * DMA_PER_WAVE * 1024;
     }
     float ex[NEL];
+    f32x4 bq[VBIAS ? 4 : 1];                 // bias / scale of the keys of registers 4 j .. 4 j + 3 (keys 32 s + 8 j + 4 hh ..)
     // score e of NEL: query block, accumulator register (the first 8 registers of every block first: they are the
     // first 16-key step of P V)
     auto el_qb = [](int e) { return QB == 2 ? (e >> 3) & 1 : 0; };
@@ -877,6 +935,11 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
           dma16_uniform_base(P == 0 ? k_src0[i] : v_src0[i], dma_off, dma_dst + i * 1024);
         }
       }
+      if constexpr (VBIAS) {
+        // (the first eight registers of every block are used in the first half of the step, the others in the second)
+        if (g == 0) { bq[0] = *(FO_LDS const f32x4*)(vbias + s * 32); bq[1] = *(FO_LDS const f32x4*)(vbias + s * 32 + 8); }
+        if (g == (GE0 + 1 + NE / 2) - 3) { bq[2] = *(FO_LDS const f32x4*)(vbias + s * 32 + 16); bq[3] = *(FO_LDS const f32x4*)(vbias + s * 32 + 24); }
+      }
       // -- this group's share of the softmax arithmetic
       if (MASK && g == GMASK) {
         // register r holds key key_base + koff(r), koff(r) = (r & 3) + 8 * (r >> 2); dead iff key > q or key >= Sk,
@@ -898,7 +961,8 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
         const int ge = GE0 + 1 + (e * NE) / NEL;
         const int b2 = el_qb(e), r = el_reg(e);
         if (ge - 1 == g) {
-          ex[e] = (DBG & 2) ? S[P][b2][r] : __builtin_fmaf(S[P][b2][r], c, -mc[b2]);
+          if constexpr (VBIAS) ex[e] = __builtin_fmaf(S[P][b2][r] + bq[r >> 2][r & 3], c, -mc[b2]);
+          else ex[e] = (DBG & 2) ? S[P][b2][r] : __builtin_fmaf(S[P][b2][r], c, -mc[b2]);
           asm volatile("" : "+v"(ex[e]));                              // pins the instruction to this micro-group
         }
         if (ge == g) {
@@ -926,15 +990,27 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
       // rare: true row maxima of this sub-tile, new references, P and row sums again, O and l rescaled
 #pragma unroll
       for (int d = 0; d < DBLK; ++d) mfma_result_fence_a(oacc[d]);
+      if constexpr (VBIAS) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          f32x4 t4 = *(FO_LDS const f32x4*)(vbias + s * 32 + 8 * j);
+          asm volatile("" : "+v"(t4));                                 // (four values at a time: no registers to spare here)
+#pragma unroll
+          for (int b2 = 0; b2 < QB; ++b2)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) S[P][b2][4 * j + u] += t4[u];
+        }
+      }
 #pragma unroll
       for (int b2 = 0; b2 < QB; ++b2) {
         float mloc = S[P][b2][0];
 #pragma unroll
         for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, S[P][b2][r]);
         mloc = fmaxf(mloc, half_swap(mloc));
-        const float m_new = fmaxf(m_run[b2], mloc);                    // finite from the first sub-tile on: key 0 is never masked
-        const float alpha = __builtin_amdgcn_exp2f((m_run[b2] - m_new) * c);
-        const float mcn = m_new * c;
+        const float m_new = fmaxf(m_run[b2], mloc);                    // finite from the first sub-tile on: key 0 is never masked ...
+        const bool no_key_yet = VBIAS && m_new == -INFINITY;           // ... but a bias may have removed every key so far
+        const float alpha = no_key_yet ? 1.0f : __builtin_amdgcn_exp2f((m_run[b2] - m_new) * c);
+        const float mcn = no_key_yet ? 0.0f : m_new * c;
         float ps = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -1021,10 +1097,16 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
     if (CAUSAL) lim = max(lim, 4 * hh - (q0w + 32 * b2 + l32));
     float mloc = -INFINITY;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : S[0][b2][r]);
+    for (int r = 0; r < 16; ++r) {
+      float sv = S[0][b2][r];
+      if constexpr (VBIAS) sv += vbias[8 * (r >> 2) + (r & 3)];
+      mloc = fmaxf(mloc, (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : sv);
+    }
     m_run[b2] = fmaxf(mloc, half_swap(mloc));
   }
-  step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1, N{});   // (its reference is its own row maximum: every P <= 1)
+  // (its reference is its own row maximum: every P <= 1 and no recovery - unless a bias removed all its keys)
+  if constexpr (VBIAS) step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1);
+  else step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1, N{});
   if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, N{}, -1);
   // Should the steps above have parked registers in scratch memory (they do not at present), wait here, visibly to
   // the compiler, for any reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0)
@@ -1142,26 +1224,27 @@ static int device_cus() {
   return n;
 }
 
-template <typename T, int D, bool CAUSAL, int QB, int DBG = 0, int BM = kWideBM>
+template <typename T, int D, bool CAUSAL, int QB, int DBG = 0, int BM = kWideBM, bool VBIAS = false>
 static int launch_wide(AttnParams p, hipStream_t stream) {
-  const size_t lds = 2 * (size_t)kRing * kBN * D * 2;
+  const size_t lds = 2 * (size_t)kRing * kBN * D * 2 + (VBIAS ? kVBiasKeys * 4 : 0);
+  if (VBIAS && (p.Sk + kBN - 1) / kBN * kBN > kVBiasKeys) return FO_ERR_UNSUPPORTED;
   p.n_qblk = (p.Sq + BM - 1) / BM;
   const unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);
   p.heavy_first = (CAUSAL && BM != kWideBM) ? heavy_first_group(p, D) : 0;
   p.order_n = 0;
-  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM, VBIAS>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
-  attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM><<<grid, BM / (32 * QB) * 64, lds, stream>>>(p);
+  attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM, VBIAS><<<grid, BM / (32 * QB) * 64, lds, stream>>>(p);
   return launch_status();
 }
 
-template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false>
+template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false, bool KBIAS = false>
 static int launch_one(const AttnParams& p, hipStream_t stream) {
-  const size_t lds_max = 4 * (size_t)kBN * D * 2 + (BIAS ? 2 * kWaves * 32 * kBN * 4 : 0);   // K, V tiles; bias tiles
-  const size_t lds = 4 * (size_t)kBN * D * 2 + (BIAS && p.bias.dma_ok ? 2 * kWaves * 32 * kBN * 4 : 0);
+  const size_t lds_max = 4 * (size_t)kBN * D * 2 + (BIAS ? 2 * kWaves * 32 * kBN * 4 : 0) + (KBIAS ? 2 * kBN * 4 : 0);   // K, V tiles; bias tiles
+  const size_t lds = 4 * (size_t)kBN * D * 2 + (BIAS && p.bias.dma_ok ? 2 * kWaves * 32 * kBN * 4 : 0) + (KBIAS ? 2 * kBN * 4 : 0);
   const unsigned grid = (unsigned)(p.n_qblk * p.B * p.H);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS, KBIAS>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max);
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
   // Order of the workgroups of one XCD when causal: the heaviest query blocks of all its heads first, then the next
@@ -1183,7 +1266,7 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
     // wherever a slot frees, and the plain order is the better one.
     const int cus_x = device_cus() / 8, n_bh_x = (int)(((int64_t)p.B * p.H) >> 3);
     const int64_t n = (int64_t)n_bh_x * p.n_qblk;
-    const int resident = (D == 64 && !DROP && !BIAS) ? 3 : 2;      // workgroups per compute unit (registers)
+    const int resident = (D == 64 && !DROP && !BIAS && !KBIAS) ? 3 : 2;      // workgroups per compute unit (registers)
     if (q.heavy_first == n_bh_x && cus_x > 0 && cus_x <= kOrderTab && n <= (int64_t)cus_x * resident && n <= kOrderTab && n > cus_x) {
       // (the table of the last shape is kept per host thread: filling it takes a few microseconds, a training loop
       // launches the same shape over and over)
@@ -1209,7 +1292,7 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
       q.order_n = (int)n;
     }
   }
-  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS><<<grid, kWaves * 64, lds, stream>>>(q);
+  attn_fwd_kernel<T, D, CAUSAL, LAZY, DBG, DROP, BIAS, KBIAS><<<grid, kWaves * 64, lds, stream>>>(q);
   return launch_status();
 }
 
@@ -1218,8 +1301,10 @@ static int launch_one(const AttnParams& p, hipStream_t stream) {
 // `forced` is the value of attn.variant (-1: the library's choice). Values from 256 on are timing ablations and exist
 // only in a build with FO_ABLATIONS.
 static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, int forced) {
-  // dropout, bias and head dims other than 64 and 128 run on the 128-row kernel
-  if (p.bias.ptr != nullptr || dropout || p.d != D) return FO_ATTN_KERNEL_ROWS128;
+  // dropout, a bias with a query stride and head dims other than 64 and 128 run on the 128-row kernel; a bias that is
+  // the same for every query (and short enough for the pipelined kernel to keep it in LDS) takes part in the choice
+  const bool key_bias = p.bias.ptr != nullptr && p.bias.strides[2] == 0 && ((int64_t)p.Sk + kBN - 1) / kBN * kBN <= kVBiasKeys;
+  if ((p.bias.ptr != nullptr && !key_bias) || dropout || p.d != D) return FO_ATTN_KERNEL_ROWS128;
   // The 256-row kernel addresses a head's keys with 32-bit byte offsets ...
   const bool wide_ok = (int64_t)p.Sk * (p.ks[2] > p.vs[2] ? p.ks[2] : p.vs[2]) * 2 < (1ll << 31);
   // ... and needs one 256-row workgroup (two query blocks each when causal) per CU to be worth it: below that the
@@ -1267,6 +1352,11 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
   }
   if (v >= 256) return v;
   if (!wide_ok && v >= FO_ATTN_KERNEL_ROWS128_PIPE) v = FO_ATTN_KERNEL_ROWS128;
+  if (key_bias) {
+    // with a bias the pipelined kernel exists in two forms: 128 rows, and 256 rows as four waves (head_dim 128)
+    if (v == FO_ATTN_KERNEL_ROWS256_W8) v = D == 128 ? FO_ATTN_KERNEL_ROWS256_W4 : FO_ATTN_KERNEL_ROWS128;
+    if (v == FO_ATTN_KERNEL_ROWS128_EXACT) v = FO_ATTN_KERNEL_ROWS128;
+  }
   if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128) v = FO_ATTN_KERNEL_ROWS128;   // the four-wave form exists for head_dim 128 only
   return v;
 }
@@ -1274,6 +1364,23 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
 template <typename T, int D>
 static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
   if (p.bias.ptr != nullptr) {
+    // A bias that is the same for every query has kernels of its own: the pipelined ones where choose_kernel says so, else
+    // the per-key form of the 128-row kernel, with or without dropout. (attn.variant 1 keeps the general bias kernel,
+    // which takes any strides: tests compare the two.)
+    if (p.bias.strides[2] == 0 && tune(g_attn_variant) != FO_ATTN_KERNEL_ROWS128_EXACT) {
+      if (!dropout) {
+        const int v = choose_kernel(p, D, causal, dropout, tune(g_attn_variant));
+        if (v >= 256) return FO_ERR_UNSUPPORTED;
+        if (v == FO_ATTN_KERNEL_ROWS128_PIPE)
+          return causal ? launch_wide<T, D, true, 1, 0, kBM, true>(p, stream) : launch_wide<T, D, false, 1, 0, kBM, true>(p, stream);
+        if constexpr (D == 128) {
+          if (v == FO_ATTN_KERNEL_ROWS256_W4)
+            return causal ? launch_wide<T, D, true, 2, 0, kWideBM, true>(p, stream) : launch_wide<T, D, false, 2, 0, kWideBM, true>(p, stream);
+        }
+        return causal ? launch_one<T, D, true, true, 0, false, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, false, true>(p, stream);
+      }
+      return causal ? launch_one<T, D, true, true, 0, true, false, true>(p, stream) : launch_one<T, D, false, true, 0, true, false, true>(p, stream);
+    }
     if (dropout) return causal ? launch_one<T, D, true, true, 0, true, true>(p, stream) : launch_one<T, D, false, true, 0, true, true>(p, stream);
     return causal ? launch_one<T, D, true, true, 0, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, true>(p, stream);
   }
@@ -1412,6 +1519,7 @@ extern "C" int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk; p.d = D;
   for (int i = 0; i < 3; ++i) { p.ks[i] = ks[i]; p.vs[i] = vs[i]; }
   p.bias.ptr = has_bias ? (const void*)ks : nullptr;   // (only tested against NULL)
+  p.bias.strides[2] = has_bias == 2 ? 0 : 1;
   return choose_kernel(p, D > 64 ? 128 : 64, causal != 0, has_dropout != 0, tune(g_attn_variant));
 }
 

@@ -86,8 +86,9 @@ int fo_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
 
 /* Which kernel fo_attn_fwd (or _dropout / _ex, with has_dropout / has_bias non-zero) launches for a call of this shape
  * on the current device with the current "attn.variant": one of the FO_ATTN_KERNEL_* codes below, or a negative
- * fo_status where fo_attn_fwd would reject the shape. Launches nothing. The choice depends on the number of compute
- * units of the device that was current when the library first chose (read once per process). No reference counterpart:
+ * fo_status where fo_attn_fwd would reject the shape. has_bias: 0 none, 1 a bias with a query stride, 2 a bias that is
+ * the same for every query (query stride 0), which the pipelined kernels take as well. Launches nothing. The choice
+ * depends on the number of compute units of the current device. No reference counterpart:
  * the reference has one kernel (flash_attention_fwd.cu:164-177); tests use this to assert which code they covered. */
 enum {
   FO_ATTN_KERNEL_ROWS128 = 0,         /* 128 query rows per workgroup, reference maximum raised lazily */

@@ -169,3 +169,179 @@ def test_bias_rejections():
     a = flash_attn(q, q, q, bias=b2)
     b = flash_attn(q, q, q, bias=b2.contiguous())
     assert torch.equal(a, b)
+
+
+# ---- a bias that is the same for every query ("1h1k", "b11k": the reference's vector bias, flash_attention_triton.py:
+# 176-186, the one its benchmark uses, benchmarks/benchmark_flash_attention.py:198) also runs in the pipelined kernels
+def _kernel_with_key_bias(B, H, Sq, Sk, D, causal, has_bias=2):
+    import ctypes
+
+    from fast_ops_amd import _lib
+
+    I3 = ctypes.c_int64 * 3
+    dense = I3(H * Sk * D, Sk * D, D)
+    code = _lib.load().fo_attn_fwd_kernel(B, H, Sq, Sk, D, dense, dense, int(causal), has_bias, 0)
+    assert code >= 0
+    return code
+
+
+@pytest.mark.parametrize("bias_dtype", ["f32", "operand"])
+@pytest.mark.parametrize("kind", ["1h1k", "b11k"])
+@pytest.mark.parametrize("case", [
+    # B, H, Sq, Sk, D, causal, kernel expected (8: 128 rows pipelined, 32: 256 rows as four waves)
+    (1, 12, 2048, 2048, 128, False, 8), (1, 12, 2048, 2048, 128, True, 8), (1, 12, 4000, 4072, 64, True, 8),
+    (2, 12, 1100, 2091, 128, False, 8), (4, 16, 2048, 2048, 128, False, 32), (2, 64, 1024, 1500, 128, True, 32),
+    (2, 8, 8192, 8192, 128, True, 32), (2, 16, 4099, 8190, 128, False, 32),
+], ids=lambda c: "-".join(str(x) for x in c))
+def test_per_key_bias_in_the_pipelined_kernels(case, kind, bias_dtype):
+    from fast_ops_amd import _lib
+
+    B, H, Sq, Sk, D, causal, expected = case
+    assert _kernel_with_key_bias(B, H, Sq, Sk, D, causal) == expected
+    assert _kernel_with_key_bias(B, H, Sq, Sk, D, causal, has_bias=1) == 0          # a bias with a query stride: plain kernel
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(Sq + Sk + D)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    k, v = (torch.randn(B, H, Sk, D, generator=g).to(dtype) for _ in range(2))
+    bias = (_bias(kind, B, H, Sq, Sk, torch.float32 if bias_dtype == "f32" else dtype, g) * 3.0)
+    qd, kd, vd, bd = (t.to(DEV) for t in (q, k, v, bias))
+    o, lse = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), causal, None, None, bd)
+    # against the oracle on some heads and query rows (the whole of the large shapes would take the CPU minutes) ...
+    heads = [(0, 0), (B - 1, H - 1)]
+    for b, h in heads:
+        rows = slice(0, Sq) if Sq * Sk <= 2048 * 2048 else slice(Sq - 700, Sq)
+        qs = q[b:b + 1, h:h + 1, rows]
+        bsl = bias[b if bias.shape[0] > 1 else 0, h if bias.shape[1] > 1 else 0][None, None].float()
+        if causal:
+            # rows of the slice keep their causal limit: the oracle masks top-left aligned, so give it the mask as bias
+            qi = torch.arange(Sq)[rows, None]
+            bsl = bsl.expand(1, 1, qs.shape[2], Sk).clone()
+            bsl[0, 0][torch.arange(Sk)[None, :] > qi] = float("-inf")
+        o_ref, lse_ref = attention_fwd_oracle(qs, k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], causal=False, bias=bsl)
+        err = (o[b, h, rows].float().cpu() - o_ref[0, 0]).abs()
+        assert float((err - (O_ATOL + O_RTOL * o_ref[0, 0].abs())).max()) <= 0, f"O head {b},{h}: max abs err {float(err.max()):.3e}"
+        assert float((lse[b, h, rows].cpu() - lse_ref[0, 0]).abs().max()) <= LSE_ATOL
+    # ... and everywhere against the plain 128-row kernel, whose bias path the tests above pin
+    _lib.tune_set("attn.variant", 0)
+    try:
+        assert _kernel_with_key_bias(B, H, Sq, Sk, D, causal) == 0
+        o0, lse0 = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), causal, None, None, bd)
+    finally:
+        _lib.tune_set("attn.variant", -1)
+    # (both round O to the operand type: one unit in the last place of the larger outputs is 2^-5)
+    assert float(((o.float() - o0.float()).abs() - (2e-2 + 2e-2 * o0.float().abs())).max()) <= 0 and float((lse - lse0).abs().max()) <= 1e-4
+    assert not torch.equal(o, torch.zeros_like(o))
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_key_padding_mask_in_the_pipelined_kernels(D, causal):
+    # -inf on the first keys (more than a tile of them: rows start without any key that counts) and on the last ones
+    B, H, S, dtype = 2, 6, 4096 if D == 64 else 2048, torch.float16
+    assert _kernel_with_key_bias(B, H, S, S, D, causal) == 8
+    g = torch.Generator().manual_seed(5 + D)
+    q, k, v = (torch.randn(B, H, S, D, generator=g).to(dtype) for _ in range(3))
+    left, right = 150, 333
+    bias = torch.zeros(B, 1, 1, S)
+    bias[0, ..., :left] = float("-inf")
+    bias[..., S - right:] = float("-inf")
+    o, lse = attn_fwd_strided(q.to(DEV), k.to(DEV), v.to(DEV), (0, 1, 2, 3), causal, None, None, bias.to(DEV))
+    for b in range(B):
+        lo = left if b == 0 else 0
+        rows = slice(lo, S)                  # causal: the rows before the first kept key have no key at all (NaN, as in attention_ref.py:59)
+        kk, vv = k[b:b + 1, :2, lo:S - right], v[b:b + 1, :2, lo:S - right]
+        if causal:
+            o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, :2, lo:S - right], kk, vv, causal=True)
+            rows = slice(lo, S - right)
+        else:
+            o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, :2, rows], kk, vv)
+        got = o[b, :2, rows].float().cpu()
+        assert torch.isfinite(got).all()
+        err = (got - o_ref[0]).abs()
+        assert float((err - (O_ATOL + O_RTOL * o_ref[0].abs())).max()) <= 0, f"batch {b}: max abs err {float(err.max()):.3e}"
+        assert float((lse[b, :2, rows].cpu() - lse_ref[0]).abs().max()) <= LSE_ATOL
+
+
+def test_per_key_bias_longer_than_the_pipelined_kernels_keep():
+    # more than 8192 keys: the row of the bias no longer fits beside the tile rings, the plain kernel takes the call
+    assert _kernel_with_key_bias(1, 12, 2048, 8256, 128, False) == 0
+    assert _kernel_with_key_bias(1, 12, 2048, 8192, 128, False) in (8, 32)
+
+
+# ---- backward with a bias that is the same for every query: the dQ kernel starts its score accumulators from it, the
+# pipelined dK/dV kernel adds one value per lane (attn_bwd.variant 0 keeps the general bias kernels pinned above)
+@pytest.mark.parametrize("bias_dtype", ["f32", "operand"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(2, 3, 200, 331, 128), (2, 3, 200, 331, 64), (1, 2, 700, 513, 128), (1, 4, 1024, 1024, 64),
+                                   (2, 2, 130, 1, 128), (1, 2, 333, 900, 40)], ids=lambda s: "x".join(map(str, s)))
+def test_backward_with_per_key_bias(shape, causal, bias_dtype):
+    from fast_ops_amd import _lib
+
+    B, H, Sq, Sk, D = shape
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(Sq * 3 + Sk + D)
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk, Sq))
+    bias = _bias("b11k" if B > 1 else "1h1k", B, H, Sq, Sk, torch.float32 if bias_dtype == "f32" else dtype, g) * 2.0
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, bias=bias)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal, bias=bias)
+    qd, kd, vd, god, bd = (t.to(DEV) for t in (q, k, v, go, bias))
+    o, lse = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), causal, None, None, bd)
+    got = attn_bwd_strided(qd, kd, vd, o, lse, god, (0, 1, 2, 3), causal, None, None, bd)
+    _check(o, lse, got, o_ref, lse_ref, ref)
+    _lib.tune_set("attn_bwd.variant", 0)
+    try:
+        other = attn_bwd_strided(qd, kd, vd, o, lse, god, (0, 1, 2, 3), causal, None, None, bd)
+    finally:
+        _lib.tune_set("attn_bwd.variant", -1)
+    for name, a, r in zip(("dQ", "dK", "dV"), got, other):
+        # (the same arithmetic up to where the bias enters the exponent: a few units in the last place of the operand type)
+        assert float(((a.float() - r.float()).abs() - (1e-2 + 2e-2 * r.float().abs())).max()) <= 0, name
+
+
+def test_backward_with_key_padding_mask_at_a_longer_shape():
+    # -inf on whole key tiles at both ends; keys that are masked get exactly zero gradients
+    B, H, S, D, dtype = 2, 2, 1500, 128, torch.float16
+    g = torch.Generator().manual_seed(77)
+    q, k, v, go = (torch.randn(B, H, S, D, generator=g).to(dtype) for _ in range(4))
+    left, right = 200, 170
+    bias = torch.zeros(B, 1, 1, S)
+    bias[..., :left] = float("-inf")
+    bias[..., S - right:] = float("-inf")
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    o, lse = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), False, None, None, bias.to(DEV))
+    dq, dk, dv = attn_bwd_strided(qd, kd, vd, o, lse, go.to(DEV), (0, 1, 2, 3), False, None, None, bias.to(DEV))
+    o_ref, lse_ref = attention_fwd_oracle(q, k[:, :, left:S - right], v[:, :, left:S - right])
+    dq_r, dk_r, dv_r = attention_bwd_oracle(q, k[:, :, left:S - right], v[:, :, left:S - right], go)
+    _check(o, lse, [dq, dk[:, :, left:S - right], dv[:, :, left:S - right]], o_ref, lse_ref, [dq_r, dk_r, dv_r])
+    for t in (dk, dv):
+        assert float(t[:, :, :left].abs().max()) == 0.0 and float(t[:, :, S - right:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("p_drop", [0.0, 0.3])
+def test_per_key_bias_in_the_128_row_kernel_with_and_without_dropout(p_drop, D, causal):
+    # small shapes stay on the 128-row kernel: its per-key form (score accumulators start from the bias) against the
+    # oracle and against the general bias kernel (attn.variant 1), forward and backward, also with dropout
+    from fast_ops_amd import _lib
+
+    B, H, Sq, Sk, dtype = 2, 3, 260, 459, torch.bfloat16
+    seed = 99
+    off = 0 if p_drop == 0 else next(o for o in range(0, 1 << 32, (1 << 20) + 777) if 0.5 < dropout_keep_mask(p_drop, seed, o, B, H, Sq, Sk).mean() < 0.9)
+    drop = None if p_drop == 0 else (p_drop, seed, off)
+    g = torch.Generator().manual_seed(D + int(causal))
+    q, k, v, go = (torch.randn(B, H, n, D, generator=g).to(dtype) for n in (Sq, Sk, Sk, Sq))
+    bias = _bias("b11k", B, H, Sq, Sk, torch.float32, g) * 2.0
+    bias[0, ..., 100:180] = float("-inf")
+    o_ref, lse_ref = attention_fwd_oracle(q, k, v, causal=causal, dropout=drop, bias=bias)
+    ref = attention_bwd_oracle(q, k, v, go, causal=causal, dropout=drop, bias=bias)
+    qd, kd, vd, god, bd = (t.to(DEV) for t in (q, k, v, go, bias))
+    o, lse = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), causal, None, drop, bd)
+    got = attn_bwd_strided(qd, kd, vd, o, lse, god, (0, 1, 2, 3), causal, None, drop, bd)
+    _check(o, lse, got, o_ref, lse_ref, ref)
+    _lib.tune_set("attn.variant", 1)
+    try:
+        o1, lse1 = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), causal, None, drop, bd)
+    finally:
+        _lib.tune_set("attn.variant", -1)
+    assert float(((o.float() - o1.float()).abs() - (2e-2 + 2e-2 * o1.float().abs())).max()) <= 0 and float((lse - lse1).abs().max()) <= 1e-4

@@ -212,6 +212,13 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     assert k(1, 12, 8192, 8192, 128, 1) == W4 and k(1, 12, 4096, 4096, 128, 0) == W4 and k(1, 12, 8192, 8192, 128, 0) == W4
     assert k(1, 10, 8192, 8192, 128, 1) == R128 and k(1, 12, 512, 512, 128, 0) == R128
     assert k(1, 12, 4096, 4096, 64, 1) == PIPE and k(1, 12, 1024, 1024, 64, 1) == R128
+    # a bias that is the same for every query (has_bias 2) takes part in the choice, with the forms that exist for it:
+    # 128 rows pipelined, 256 rows as four waves (head_dim 128), the 128-row kernel; a bias with a query stride does not
+    assert k(1, 12, 2048, 2048, 128, 1, bias=2) == PIPE and k(1, 12, 2048, 2048, 128, 1, bias=1) == R128
+    assert k(2, 16, 8192, 8192, 128, 1, bias=2) == W4 and k(2, 16, 4096, 4096, 128, 1, bias=2) == W4    # (W8 without bias)
+    assert k(1, 8, 8192, 8192, 64, 0, bias=2) == R128 and k(1, 12, 4096, 4096, 64, 1, bias=2) == PIPE
+    assert k(2, 16, 8192, 8256, 128, 0, bias=2) == R128 and k(2, 16, 8192, 8130, 128, 0, bias=2) == W4  # at most 8192 keys in LDS
+    assert k(2, 16, 8192, 8192, 128, 1, bias=2, drop=1) == R128
     # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
     assert k(2, 16, 8192, 8192, 96, 1) == _lib.FO_ATTN_KERNEL_ROWS128
     assert lib.fo_attn_fwd_kernel(1, 1, 128, 128, 64, None, dense(128, 64), 0, 0, 0) == -1
