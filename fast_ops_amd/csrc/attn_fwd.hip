@@ -1326,10 +1326,13 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // head_dim 128, causal: from 1024 queries on (B*H = 128: 1024 queries -8 %, 1536 -16 %, 2048 -12 % against the
     // 128-row kernel; 512 and 768 queries +7 % and +18 %, a 256-row block being a large part of so small a triangle).
     if (D == 128 && causal && p.Sq < 1024) wide = false;
-    // head_dim 64 (half the MFMAs per score, so the softmax weighs twice as much and the 128-row kernel's two workgroups
-    // per CU hide it better): only for long rows of keys. Non-causal 1024 keys +20 %, 2048 +5 %, 4096 +0.6 %, 8192
-    // -0.5 %, 16384 -1.8 %; causal 2048 +10 %, 4096 +6.6 %, 6144 +5.5 %, 8192 +1.5 %, 16384 -1.2 %.
-    if (D == 64 && keys < (causal ? 16384 : 8192)) wide = false;
+    // head_dim 64 (half the MFMAs per score, so the softmax weighs twice as much and the 128-row kernel's workgroups
+    // sharing a CU hide it better): only for long rows of keys, and as four waves x 64 rows, which halves the LDS reads
+    // per MFMA (on random operands this head_dim too runs at the clock the power budget leaves: all-zero operands take
+    // 28 % less time). Four-wave form against the 128-row kernel: non-causal 1024 keys +2 %, 2048 -3 %, 4096 -6 %,
+    // 8192 -6.5 %, 16384 -6 %; causal 2048 +3 %, 4096 -2 %, 8192 -5 %, 16384 -8 %. (The eight-wave form is 4-5 % behind
+    // the four-wave form everywhere: non-causal 1024 keys +20 %, 4096 +0.6 %, 16384 -1.8 % against the 128-row kernel.)
+    if (D == 64 && keys < (causal ? 8192 : 4096)) wide = false;
     v = wide ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128;
     // Few workgroups for the chip (12 heads of a tensor-parallel split, short batches): what bounds the launch then is
     // the time a workgroup takes per key tile, not throughput, and 128-row workgroups in the pipelined kernel take less
@@ -1348,7 +1351,7 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // tile, and its longer pipeline fill and drain have to be spread over enough tiles. Measured on one box, new form
     // against the eight-wave form: non-causal 2048 keys -1.0 %, 4096 -2.3 %, 8192 -2.5 %; causal 3072 +3 %, 4096 +1 %,
     // 8192 -0.7 %, 16384 -1.8 %.
-    if (v == FO_ATTN_KERNEL_ROWS256_W8 && D == 128 && keys >= (causal ? 6144 : 2048)) v = FO_ATTN_KERNEL_ROWS256_W4;
+    if (v == FO_ATTN_KERNEL_ROWS256_W8 && (D == 64 || keys >= (causal ? 6144 : 2048))) v = FO_ATTN_KERNEL_ROWS256_W4;
   }
   if (v >= 256) return v;
   if (!wide_ok && v >= FO_ATTN_KERNEL_ROWS128_PIPE) v = FO_ATTN_KERNEL_ROWS128;
@@ -1357,7 +1360,7 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     if (v == FO_ATTN_KERNEL_ROWS256_W8) v = D == 128 ? FO_ATTN_KERNEL_ROWS256_W4 : FO_ATTN_KERNEL_ROWS128;
     if (v == FO_ATTN_KERNEL_ROWS128_EXACT) v = FO_ATTN_KERNEL_ROWS128;
   }
-  if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128) v = FO_ATTN_KERNEL_ROWS128;   // the four-wave form exists for head_dim 128 only
+  if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128 && key_bias) v = FO_ATTN_KERNEL_ROWS128;   // (with a bias: head_dim 128 only)
   return v;
 }
 
@@ -1388,9 +1391,7 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
   const int v = choose_kernel(p, D, causal, dropout, tune(g_attn_variant));
   if (v == FO_ATTN_KERNEL_ROWS256_W8) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
   if (v == FO_ATTN_KERNEL_ROWS128_PIPE) return causal ? launch_wide<T, D, true, 1, 0, kBM>(p, stream) : launch_wide<T, D, false, 1, 0, kBM>(p, stream);
-  if constexpr (D == 128) {
-    if (v == FO_ATTN_KERNEL_ROWS256_W4) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
-  }
+  if (v == FO_ATTN_KERNEL_ROWS256_W4) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
 #if defined(FO_ABLATIONS)
   // Timing ablations (WRONG results by design; bf16, head_dim 128 only). 256-row kernel, non-causal: 256 + bits for eight
   // waves, 512 + bits for four; bit 0 no global->LDS copies, 1 no exponentials, 2 no LDS fragment reads, 5 no wait for

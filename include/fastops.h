@@ -95,7 +95,7 @@ enum {
   FO_ATTN_KERNEL_ROWS128_EXACT = 1,   /* the same with the exact running maximum of flash_attention_triton.py:200-213 */
   FO_ATTN_KERNEL_ROWS128_PIPE = 8,    /* 128 query rows per workgroup, four waves x 32 rows, in the 256-row kernel's pipeline */
   FO_ATTN_KERNEL_ROWS256_W8 = 16,     /* 256 query rows per workgroup, eight waves x 32 rows */
-  FO_ATTN_KERNEL_ROWS256_W4 = 32      /* 256 query rows per workgroup, four waves x 64 rows (head_dim 128 only) */
+  FO_ATTN_KERNEL_ROWS256_W4 = 32      /* 256 query rows per workgroup, four waves x 64 rows */
 };
 int fo_attn_fwd_kernel(int B, int H, int Sq, int Sk, int D, const int64_t* k_strides_host, const int64_t* v_strides_host,
                        int causal, int has_bias, int has_dropout);

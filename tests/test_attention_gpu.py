@@ -42,7 +42,7 @@ def _check(o, lse, o_ref, lse_ref, what=""):
 
 # attn.variant values: -1 = the library's choice (which depends on head_dim and on how many workgroups the shape gives),
 # 8 = 128 rows per workgroup in the pipelined kernel (four waves x 32 rows),
-# 0 = the 128-row kernel, 16 / 32 = the 256-row kernel with eight / four waves (four: head_dim 128 only)
+# 0 = the 128-row kernel, 16 / 32 = the 256-row kernel with eight / four waves
 KERNELS_D128 = [-1, 0, 8, 16, 32]
 
 
@@ -205,8 +205,6 @@ def test_headline_shape_on_both_forms_of_the_256_row_kernel(kernel_variant):
 def test_256_row_kernel_with_heads_dealt_to_xcds_and_several_items_per_head(shape, causal, D, kernel_variant):
     # 8, 16 and 24 heads (a multiple of the 8 XCDs: workgroup id -> (XCD, head, item)) with 3 to 7 items per head, ragged
     # lengths; causal items are pairs of query blocks, the middle one single when their number is odd
-    if D == 64 and kernel_variant == 32:
-        pytest.skip("head_dim 64 has no four-wave form of the 256-row kernel")
     B, H, Sq, Sk = shape
     q, k, v = _qkv(B, H, Sq, Sk, D, torch.bfloat16, seed=Sq + Sk + D)
     assert _kernel_taken(q, k, v, causal) == kernel_variant
@@ -219,8 +217,6 @@ def test_256_row_kernel_with_heads_dealt_to_xcds_and_several_items_per_head(shap
 @pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
 def test_ragged_and_unequal_lengths(shape, causal, D, kernel_variant):
     # sequence lengths that are not multiples of the 128-row / 64-key tiles, Sq != Sk (causal mask is top-left aligned)
-    if D == 64 and kernel_variant == 32:
-        pytest.skip("head_dim 64 has no four-wave form of the 256-row kernel")
     B, H, Sq, Sk = shape
     _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
 
@@ -238,19 +234,19 @@ def test_ragged_across_256_row_blocks_and_ring_wraps(shape, causal, dtype, kerne
 @pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
-@pytest.mark.parametrize("kernel_variant", [-1, 0, 8, 16], indirect=True)
+@pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
 def test_ragged_across_256_row_blocks_head_dim_64(shape, causal, dtype, kernel_variant):
     B, H, Sq, Sk = shape
     _run_and_check(B, H, Sq, Sk, 64, dtype, causal, seed=Sq + Sk + 64)
 
 
-@pytest.mark.parametrize("causal,S", [(True, 16384), (False, 8192)])
-def test_head_dim_64_long_shape_takes_the_256_row_kernel_by_default(causal, S):
-    # head_dim 64 takes the 256-row kernel only for long rows of keys (8192 non-causal, 16384 causal) and one workgroup
-    # per CU (8 heads x 32 blocks / pairs of blocks): the library's own choice, and it must agree with the oracle
-    q, k, v = _qkv(1, 8, S, S, 64, torch.bfloat16, seed=5)
-    assert _kernel_taken(q, k, v, causal) == _lib.FO_ATTN_KERNEL_ROWS256_W8
-    _run_and_check(1, 8, S, S, 64, torch.bfloat16, causal, seed=5)
+@pytest.mark.parametrize("causal,S,heads", [(True, 16384, 8), (True, 8192, 16), (False, 8192, 8), (False, 4096, 16)])
+def test_head_dim_64_long_shape_takes_the_256_row_kernel_by_default(causal, S, heads):
+    # head_dim 64 takes the 256-row kernel, as four waves x 64 rows, only for long rows of keys (from 4096 non-causal,
+    # 8192 causal) and at least one workgroup per CU: the library's own choice, and it must agree with the oracle
+    q, k, v = _qkv(1, heads, S, S, 64, torch.bfloat16, seed=5)
+    assert _kernel_taken(q, k, v, causal) == _lib.FO_ATTN_KERNEL_ROWS256_W4
+    _run_and_check(1, heads, S, S, 64, torch.bfloat16, causal, seed=5)
 
 
 @pytest.mark.parametrize("causal,S", [(True, 2304), (False, 1024)])
@@ -290,8 +286,6 @@ def test_causal_up_to_2048_queries_takes_the_128_row_kernel_by_default():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
 @pytest.mark.parametrize("kernel_variant", KERNELS_D128, indirect=True)
 def test_moving_row_maximum(pattern, causal, D, dtype, kernel_variant):
-    if D == 64 and kernel_variant == 32:
-        pytest.skip("head_dim 64 has no four-wave form of the 256-row kernel")
     # scores whose row maximum keeps moving (or sits far above the rest) exercise the rescaling of the running
     # softmax state: keys scaled so that scaled scores span tens of units
     B, H, Sq, Sk = 1, 2, 384, 640

@@ -185,7 +185,7 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     assert lib.fo_tune_set(b"attn.variant", 32) == 0
     try:
         assert k(1, 1, 512, 512, 128, 0) == _lib.FO_ATTN_KERNEL_ROWS256_W4
-        assert k(1, 1, 512, 512, 64, 0) == _lib.FO_ATTN_KERNEL_ROWS128          # no four-wave form for head_dim 64
+        assert k(1, 1, 512, 512, 64, 0) == _lib.FO_ATTN_KERNEL_ROWS256_W4
         assert lib.fo_tune_set(b"attn.variant", 1) == 0
         assert k(1, 1, 512, 512, 64, 1) == _lib.FO_ATTN_KERNEL_ROWS128_EXACT
     finally:
@@ -204,8 +204,8 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     assert k(12, 16, 1024, 1024, 128, 1) == R128         # 384 workgroups would leave half of the second round empty
     assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
     assert k(16, 16, 512, 512, 128, 0) == W8 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups
-    assert k(1, 8, 8192, 8192, 64, 0) == W8 and k(4, 8, 4096, 4096, 64, 0) == R128     # head_dim 64: long rows only
-    assert k(1, 8, 16384, 16384, 64, 1) == W8 and k(2, 16, 8192, 8192, 64, 1) == R128
+    assert k(1, 8, 8192, 8192, 64, 0) == W4 and k(4, 8, 4096, 4096, 64, 0) == W4 and k(8, 8, 2048, 2048, 64, 0) == R128   # head_dim 64: long rows only,
+    assert k(1, 8, 16384, 16384, 64, 1) == W4 and k(2, 16, 8192, 8192, 64, 1) == W4 and k(4, 16, 4096, 4096, 64, 1) == R128  # and four waves
     # too few workgroups for the chip (12 heads of a tensor-parallel split): 128-row workgroups in the pipelined kernel
     assert k(1, 12, 2048, 2048, 128, 1) == PIPE and k(1, 12, 2048, 2048, 128, 0) == PIPE and k(1, 12, 4096, 4096, 128, 1) == PIPE
     # long rows of keys at head_dim 128: the 256-row kernel already with three quarters of one round of workgroups
