@@ -104,29 +104,40 @@ def _time_steps(step, steps, warmup, settle=0, before_each=None, wall_without_ev
     given, runs before timed step i outside its pair of events (fresh inputs for the step). With `wall_without_events`
     the wall time per step comes from K further steps with no events between them (for kernels of a few tens of
     microseconds, where the two event records per step are a sizeable part of a step)."""
+    import gc
+
     import torch
 
     info = _settle(step, settle)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    wall_plain = None
-    if wall_without_events:
+    # (Python's cycle collector stays out of the timed steps: a full collection in this process takes tens of
+    # milliseconds of host time, which the events around a 30-microsecond launch see as the GPU waiting)
+    gc.collect()
+    gc_was_on = gc.isenabled()
+    gc.disable()
+    try:
+        wall_plain = None
+        if wall_without_events:
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            wall_plain = (time.perf_counter() - t0) * 1e3 / steps
+        starts, ends = _events(steps), _events(steps)
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for i in range(steps):
+            if before_each is not None:
+                before_each(i)
+            starts[i].record()
             step()
+            ends[i].record()
         torch.cuda.synchronize()
-        wall_plain = (time.perf_counter() - t0) * 1e3 / steps
-    starts, ends = _events(steps), _events(steps)
-    t0 = time.perf_counter()
-    for i in range(steps):
-        if before_each is not None:
-            before_each(i)
-        starts[i].record()
-        step()
-        ends[i].record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
+        wall_ms = (time.perf_counter() - t0) * 1e3
+    finally:
+        if gc_was_on:
+            gc.enable()
     per_launch = [starts[i].elapsed_time(ends[i]) for i in range(steps)]
     info = dict(info, kernel_ms_median=sorted(per_launch)[steps // 2])
     return (wall_plain if wall_plain is not None else wall_ms / steps), sum(per_launch) / steps, min(per_launch), info

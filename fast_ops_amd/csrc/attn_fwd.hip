@@ -1356,11 +1356,10 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
   if (v >= 256) return v;
   if (!wide_ok && v >= FO_ATTN_KERNEL_ROWS128_PIPE) v = FO_ATTN_KERNEL_ROWS128;
   if (key_bias) {
-    // with a bias the pipelined kernel exists in two forms: 128 rows, and 256 rows as four waves (head_dim 128)
-    if (v == FO_ATTN_KERNEL_ROWS256_W8) v = D == 128 ? FO_ATTN_KERNEL_ROWS256_W4 : FO_ATTN_KERNEL_ROWS128;
+    // with a bias the pipelined kernel exists in two forms: 128 rows, and 256 rows as four waves
+    if (v == FO_ATTN_KERNEL_ROWS256_W8) v = FO_ATTN_KERNEL_ROWS256_W4;
     if (v == FO_ATTN_KERNEL_ROWS128_EXACT) v = FO_ATTN_KERNEL_ROWS128;
   }
-  if (v == FO_ATTN_KERNEL_ROWS256_W4 && D != 128 && key_bias) v = FO_ATTN_KERNEL_ROWS128;   // (with a bias: head_dim 128 only)
   return v;
 }
 
@@ -1376,10 +1375,8 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
         if (v >= 256) return FO_ERR_UNSUPPORTED;
         if (v == FO_ATTN_KERNEL_ROWS128_PIPE)
           return causal ? launch_wide<T, D, true, 1, 0, kBM, true>(p, stream) : launch_wide<T, D, false, 1, 0, kBM, true>(p, stream);
-        if constexpr (D == 128) {
-          if (v == FO_ATTN_KERNEL_ROWS256_W4)
-            return causal ? launch_wide<T, D, true, 2, 0, kWideBM, true>(p, stream) : launch_wide<T, D, false, 2, 0, kWideBM, true>(p, stream);
-        }
+        if (v == FO_ATTN_KERNEL_ROWS256_W4)
+          return causal ? launch_wide<T, D, true, 2, 0, kWideBM, true>(p, stream) : launch_wide<T, D, false, 2, 0, kWideBM, true>(p, stream);
         return causal ? launch_one<T, D, true, true, 0, false, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, false, true>(p, stream);
       }
       return causal ? launch_one<T, D, true, true, 0, true, false, true>(p, stream) : launch_one<T, D, false, true, 0, true, false, true>(p, stream);

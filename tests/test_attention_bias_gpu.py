@@ -191,7 +191,7 @@ def _kernel_with_key_bias(B, H, Sq, Sk, D, causal, has_bias=2):
     # B, H, Sq, Sk, D, causal, kernel expected (8: 128 rows pipelined, 32: 256 rows as four waves)
     (1, 12, 2048, 2048, 128, False, 8), (1, 12, 2048, 2048, 128, True, 8), (1, 12, 4000, 4072, 64, True, 8),
     (2, 12, 1100, 2091, 128, False, 8), (4, 16, 2048, 2048, 128, False, 32), (2, 64, 1024, 1500, 128, True, 32),
-    (2, 8, 8192, 8192, 128, True, 32), (2, 16, 4099, 8190, 128, False, 32),
+    (2, 8, 8192, 8192, 128, True, 32), (2, 16, 4099, 8190, 128, False, 32), (4, 8, 4096, 4100, 64, False, 32), (2, 16, 8192, 8192, 64, True, 32),
 ], ids=lambda c: "-".join(str(x) for x in c))
 def test_per_key_bias_in_the_pipelined_kernels(case, kind, bias_dtype):
     from fast_ops_amd import _lib

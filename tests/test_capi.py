@@ -216,7 +216,7 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     # 128 rows pipelined, 256 rows as four waves (head_dim 128), the 128-row kernel; a bias with a query stride does not
     assert k(1, 12, 2048, 2048, 128, 1, bias=2) == PIPE and k(1, 12, 2048, 2048, 128, 1, bias=1) == R128
     assert k(2, 16, 8192, 8192, 128, 1, bias=2) == W4 and k(2, 16, 4096, 4096, 128, 1, bias=2) == W4    # (W8 without bias)
-    assert k(1, 8, 8192, 8192, 64, 0, bias=2) == R128 and k(1, 12, 4096, 4096, 64, 1, bias=2) == PIPE
+    assert k(1, 8, 8192, 8192, 64, 0, bias=2) == W4 and k(1, 12, 4096, 4096, 64, 1, bias=2) == PIPE
     assert k(2, 16, 8192, 8256, 128, 0, bias=2) == R128 and k(2, 16, 8192, 8130, 128, 0, bias=2) == W4  # at most 8192 keys in LDS
     assert k(2, 16, 8192, 8192, 128, 1, bias=2, drop=1) == R128
     # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
