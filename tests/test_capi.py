@@ -194,31 +194,36 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
     # the query refuses what the call refuses: sizes beyond the launch limits, strides that are negative or no multiple of 8
     assert k(1 << 15, 1 << 15, 1 << 12, 128, 64, 0) == -4 and k(1 << 10, 1 << 10, 1 << 21, 128, 64, 0) == -4
     assert k(1, 1, 128, 128, 64, 0, ks=I3(0, -8, 64)) == -5 and k(1, 1, 128, 128, 64, 0, ks=I3(0, 12, 64)) == -5
-    # the library's own choice on 256 CUs (an MI355X, or what the library assumes where it finds no device)
+    # the library's own choice on 256 CUs (an MI355X, or what the library assumes where it finds no device); on a device
+    # with another number of compute units the thresholds move, and the expectations below do not apply
+    import torch
+
+    on_256_cus = not torch.cuda.is_available() or torch.cuda.get_device_properties(0).multi_processor_count == 256
     R128, W8, W4, PIPE = _lib.FO_ATTN_KERNEL_ROWS128, _lib.FO_ATTN_KERNEL_ROWS256_W8, _lib.FO_ATTN_KERNEL_ROWS256_W4, _lib.FO_ATTN_KERNEL_ROWS128_PIPE
-    assert k(2, 16, 8192, 8192, 128, 1) == W4            # the headline shape: 512 workgroups of two query blocks
-    assert k(16, 32, 2048, 2048, 128, 0) == W4           # B=16 H=32 S=2048 non-causal
-    assert k(8, 12, 1024, 1024, 64, 1) == R128           # the GPT-2-small shape
-    assert k(2, 16, 4096, 4096, 128, 1) == W8            # fewer than 6144 keys, causal: eight waves
-    assert k(8, 16, 1024, 1024, 128, 1) == W8            # causal from 1024 queries on: 256 workgroups, one round
-    assert k(12, 16, 1024, 1024, 128, 1) == R128         # 384 workgroups would leave half of the second round empty
-    assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
-    assert k(16, 16, 512, 512, 128, 0) == W8 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups
-    assert k(1, 8, 8192, 8192, 64, 0) == W4 and k(4, 8, 4096, 4096, 64, 0) == W4 and k(8, 8, 2048, 2048, 64, 0) == R128   # head_dim 64: long rows only,
-    assert k(1, 8, 16384, 16384, 64, 1) == W4 and k(2, 16, 8192, 8192, 64, 1) == W4 and k(4, 16, 4096, 4096, 64, 1) == R128  # and four waves
-    # too few workgroups for the chip (12 heads of a tensor-parallel split): 128-row workgroups in the pipelined kernel
-    assert k(1, 12, 2048, 2048, 128, 1) == PIPE and k(1, 12, 2048, 2048, 128, 0) == PIPE and k(1, 12, 4096, 4096, 128, 1) == PIPE
-    # long rows of keys at head_dim 128: the 256-row kernel already with three quarters of one round of workgroups
-    assert k(1, 12, 8192, 8192, 128, 1) == W4 and k(1, 12, 4096, 4096, 128, 0) == W4 and k(1, 12, 8192, 8192, 128, 0) == W4
-    assert k(1, 10, 8192, 8192, 128, 1) == R128 and k(1, 12, 512, 512, 128, 0) == R128
-    assert k(1, 12, 4096, 4096, 64, 1) == PIPE and k(1, 12, 1024, 1024, 64, 1) == R128
-    # a bias that is the same for every query (has_bias 2) takes part in the choice, with the forms that exist for it:
-    # 128 rows pipelined, 256 rows as four waves (head_dim 128), the 128-row kernel; a bias with a query stride does not
-    assert k(1, 12, 2048, 2048, 128, 1, bias=2) == PIPE and k(1, 12, 2048, 2048, 128, 1, bias=1) == R128
-    assert k(2, 16, 8192, 8192, 128, 1, bias=2) == W4 and k(2, 16, 4096, 4096, 128, 1, bias=2) == W4    # (W8 without bias)
-    assert k(1, 8, 8192, 8192, 64, 0, bias=2) == W4 and k(1, 12, 4096, 4096, 64, 1, bias=2) == PIPE
-    assert k(2, 16, 8192, 8256, 128, 0, bias=2) == R128 and k(2, 16, 8192, 8130, 128, 0, bias=2) == W4  # at most 8192 keys in LDS
-    assert k(2, 16, 8192, 8192, 128, 1, bias=2, drop=1) == R128
+    if on_256_cus:
+        assert k(2, 16, 8192, 8192, 128, 1) == W4            # the headline shape: 512 workgroups of two query blocks
+        assert k(16, 32, 2048, 2048, 128, 0) == W4           # B=16 H=32 S=2048 non-causal
+        assert k(8, 12, 1024, 1024, 64, 1) == R128           # the GPT-2-small shape
+        assert k(2, 16, 4096, 4096, 128, 1) == W8            # fewer than 6144 keys, causal: eight waves
+        assert k(8, 16, 1024, 1024, 128, 1) == W8            # causal from 1024 queries on: 256 workgroups, one round
+        assert k(12, 16, 1024, 1024, 128, 1) == R128         # 384 workgroups would leave half of the second round empty
+        assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
+        assert k(16, 16, 512, 512, 128, 0) == W8 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups
+        assert k(1, 8, 8192, 8192, 64, 0) == W4 and k(4, 8, 4096, 4096, 64, 0) == W4 and k(8, 8, 2048, 2048, 64, 0) == R128   # head_dim 64: long rows only,
+        assert k(1, 8, 16384, 16384, 64, 1) == W4 and k(2, 16, 8192, 8192, 64, 1) == W4 and k(4, 16, 4096, 4096, 64, 1) == R128  # and four waves
+        # too few workgroups for the chip (12 heads of a tensor-parallel split): 128-row workgroups in the pipelined kernel
+        assert k(1, 12, 2048, 2048, 128, 1) == PIPE and k(1, 12, 2048, 2048, 128, 0) == PIPE and k(1, 12, 4096, 4096, 128, 1) == PIPE
+        # long rows of keys at head_dim 128: the 256-row kernel already with three quarters of one round of workgroups
+        assert k(1, 12, 8192, 8192, 128, 1) == W4 and k(1, 12, 4096, 4096, 128, 0) == W4 and k(1, 12, 8192, 8192, 128, 0) == W4
+        assert k(1, 10, 8192, 8192, 128, 1) == R128 and k(1, 12, 512, 512, 128, 0) == R128
+        assert k(1, 12, 4096, 4096, 64, 1) == PIPE and k(1, 12, 1024, 1024, 64, 1) == R128
+        # a bias that is the same for every query (has_bias 2) takes part in the choice, with the forms that exist for it:
+        # 128 rows pipelined, 256 rows as four waves (head_dim 128), the 128-row kernel; a bias with a query stride does not
+        assert k(1, 12, 2048, 2048, 128, 1, bias=2) == PIPE and k(1, 12, 2048, 2048, 128, 1, bias=1) == R128
+        assert k(2, 16, 8192, 8192, 128, 1, bias=2) == W4 and k(2, 16, 4096, 4096, 128, 1, bias=2) == W4    # (W8 without bias)
+        assert k(1, 8, 8192, 8192, 64, 0, bias=2) == W4 and k(1, 12, 4096, 4096, 64, 1, bias=2) == PIPE
+        assert k(2, 16, 8192, 8256, 128, 0, bias=2) == R128 and k(2, 16, 8192, 8130, 128, 0, bias=2) == W4  # at most 8192 keys in LDS
+        assert k(2, 16, 8192, 8192, 128, 1, bias=2, drop=1) == R128
     # head dims other than 64 and 128 take the 128-row kernel, whatever is forced
     assert k(2, 16, 8192, 8192, 96, 1) == _lib.FO_ATTN_KERNEL_ROWS128
     assert lib.fo_attn_fwd_kernel(1, 1, 128, 128, 64, None, dense(128, 64), 0, 0, 0) == -1
