@@ -345,3 +345,35 @@ def test_per_key_bias_in_the_128_row_kernel_with_and_without_dropout(p_drop, D, 
     finally:
         _lib.tune_set("attn.variant", -1)
     assert float(((o.float() - o1.float()).abs() - (2e-2 + 2e-2 * o1.float().abs())).max()) <= 0 and float((lse - lse1).abs().max()) <= 1e-4
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_per_key_bias_properties_at_the_headline_size(causal):
+    # B=2 H=16 S=8192 D=128 bf16 (the 256-row kernel with the bias row in LDS), by what the mathematics fixes: a bias that
+    # is the same for every key changes nothing but LSE, which moves by that constant; -inf on the last keys is attention
+    # over the keys before them; and the backward of both agrees with the backward without bias
+    B, H, S, D, dtype = 2, 16, 8192, 128, torch.bfloat16
+    assert _kernel_with_key_bias(B, H, S, S, D, causal) == 32
+    g = torch.Generator().manual_seed(123)
+    q, k, v, go = (torch.randn(B, H, S, D, generator=g).to(dtype).to(DEV) for _ in range(4))
+    dims = (0, 1, 2, 3)
+    o0, lse0 = attn_fwd_strided(q, k, v, dims, causal, None, None, None)
+    const = torch.full((B, 1, 1, S), 1.75, device=DEV)
+    o1, lse1 = attn_fwd_strided(q, k, v, dims, causal, None, None, const)
+    assert float((o1.float() - o0.float()).abs().max()) <= 2e-2 and float((lse1 - lse0 - 1.75).abs().max()) <= 1e-3
+    cut = 5000
+    pad = torch.zeros(B, 1, 1, S, device=DEV)
+    pad[..., cut:] = float("-inf")
+    o2, lse2 = attn_fwd_strided(q, k, v, dims, causal, None, None, pad)
+    o3, lse3 = attn_fwd_strided(q, k[:, :, :cut], v[:, :, :cut], dims, causal, None, None, None)
+    assert float((o2.float() - o3.float()).abs().max()) <= 2e-2 and float((lse2 - lse3).abs().max()) <= 1e-3
+    d0 = attn_bwd_strided(q, k, v, o0, lse0, go, dims, causal, None, None, None)
+    d1 = attn_bwd_strided(q, k, v, o1, lse1, go, dims, causal, None, None, const)
+    d2 = attn_bwd_strided(q, k, v, o2, lse2, go, dims, causal, None, None, pad)
+    d3 = attn_bwd_strided(q, k[:, :, :cut], v[:, :, :cut], o3, lse3, go, dims, causal, None, None, None)
+    for name, a, b_ in zip(("dQ", "dK", "dV"), d1, d0):
+        assert float((a.float() - b_.float()).abs().max()) <= 2e-2 * max(1.0, float(b_.float().abs().max())), name
+    assert float((d2[0].float() - d3[0].float()).abs().max()) <= 2e-2 * max(1.0, float(d3[0].float().abs().max()))
+    for a, b_ in ((d2[1], d3[1]), (d2[2], d3[2])):
+        assert float((a[:, :, :cut].float() - b_.float()).abs().max()) <= 2e-2 * max(1.0, float(b_.float().abs().max()))
+        assert float(a[:, :, cut:].abs().max()) == 0.0
