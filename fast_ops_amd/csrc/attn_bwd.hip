@@ -165,6 +165,54 @@ __device__ __forceinline__ void copy_tile64_inside(const T* base, int64_t stride
   for (int i = 0; i < TileLaneOffsets<T, D>::N; ++i) dma16_uniform_base(tile, lo.off[i], dst + (wave_s * TileLaneOffsets<T, D>::N + i) * 1024);
 }
 
+// The same offsets kept as two registers per matrix instead of one per piece, for a kernel that has none to spare: the
+// byte offset of the lane's row of piece 0 and of its 16-byte chunk in that row. Piece i lies ROWS_PER_DMA * i rows
+// further (added to the uniform base) and its rows' swizzle differs from piece 0's in fixed bits (i for 256-byte rows,
+// 2 i for 128-byte rows: the bits of the row number that the swizzle takes and the piece index changes), so a piece's
+// offset is an XOR with a constant and an addition.
+template <typename T, int D>
+struct TileLaneOffsetsCompact {
+  static constexpr int N = kBwdTile * D * 2 / 1024 / kBwdWaves;
+  static constexpr int ROW_BYTES = D * 2, CHUNKS = ROW_BYTES / 16, ROWS_PER_DMA = 1024 / ROW_BYTES;
+  uint32_t row_bytes0, chunk_bytes0;
+  bool ok;
+  __device__ __forceinline__ void init(int64_t stride, int d, int wave_s, int lane) {
+    ok = stride < (1 << 23) && d == D;
+    const int row = (wave_s * N) * ROWS_PER_DMA + lane / CHUNKS;
+    row_bytes0 = (uint32_t)(row * (int)stride) * 2u;
+    chunk_bytes0 = (uint32_t)(((lane % CHUNKS) ^ swz<D>(row)) * 16);
+  }
+  static constexpr uint32_t flip(int i) { return (uint32_t)((D == 128 ? i : 2 * i) * 16); }
+  // (wave_s * N is a multiple of N = 4 or 2, so the piece index occupies bits of the row number that are zero in piece 0)
+  static_assert((D == 128 && N == 4) || (D == 64 && N == 2), "which bits of the swizzle a piece index changes");
+};
+// Two tiles (K and V) at once: every offset is computed before the first copy goes out. (Should the compiler have parked
+// one of the four registers in scratch memory, its reload - which it waits for with vmcnt(0) - then comes before the
+// copies and finds nothing in flight; between two copies it would wait for the first one to land.)
+template <typename T, int D>
+__device__ __forceinline__ void copy_two_tiles64_inside(const T* base_a, int64_t stride_a, const TileLaneOffsetsCompact<T, D>& lo_a, FO_LDS char* dst_a,
+                                                        const T* base_b, int64_t stride_b, const TileLaneOffsetsCompact<T, D>& lo_b, FO_LDS char* dst_b,
+                                                        int row0, int wave_s) {
+  typedef TileLaneOffsetsCompact<T, D> L;
+  const char* tile_a = (const char*)(base_a + (int64_t)row0 * stride_a);
+  const char* tile_b = (const char*)(base_b + (int64_t)row0 * stride_b);
+  uint32_t ra = lo_a.row_bytes0, ca = lo_a.chunk_bytes0, rb = lo_b.row_bytes0, cb = lo_b.chunk_bytes0;
+  // (recomputed per tile: hoisted out of the loop they would be 2 N registers again)
+  asm volatile("" : "+v"(ra), "+v"(ca), "+v"(rb), "+v"(cb));
+  uint32_t off_a[L::N], off_b[L::N];
+#pragma unroll
+  for (int i = 0; i < L::N; ++i) {
+    off_a[i] = ra + (ca ^ L::flip(i));
+    off_b[i] = rb + (cb ^ L::flip(i));
+    asm volatile("" : "+v"(off_a[i]), "+v"(off_b[i]));
+  }
+#pragma unroll
+  for (int i = 0; i < L::N; ++i) {
+    dma16_uniform_base(tile_a + (int64_t)i * L::ROWS_PER_DMA * stride_a * 2, off_a[i], dst_a + (wave_s * L::N + i) * 1024);
+    dma16_uniform_base(tile_b + (int64_t)i * L::ROWS_PER_DMA * stride_b * 2, off_b[i], dst_b + (wave_s * L::N + i) * 1024);
+  }
+}
+
 // A operand of a 32x32x16 MFMA from a row-major tile in LDS: lane = row l32 of block `blk`, 8 elements at
 // column 16*ks + 8*hh
 template <typename T, int D>
@@ -246,7 +294,10 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   const T* vbase = (const T*)prm.v + b * prm.vs[0] + h * prm.vs[1];
   const int n_tiles = CAUSAL ? (min(Sk, q0 + kBwdRows) + kBwdTile - 1) / kBwdTile : (Sk + kBwdTile - 1) / kBwdTile;
 
-  TileLaneOffsets<T, D> klo, vlo;
+  // (one register per piece where the kernel has them - head_dim 64, and the plain causal form at head_dim 128, which
+  // were 0.4-0.6 % faster that way - and two per matrix where it would otherwise park some in scratch memory)
+  constexpr bool ROOMY = D == 64 || (CAUSAL && !DROP && !BIAS && !KBIAS);
+  typename std::conditional<ROOMY, TileLaneOffsets<T, D>, TileLaneOffsetsCompact<T, D>>::type klo, vlo;
   klo.init(prm.ks[2], prm.d, wave_s, lane);
   vlo.init(prm.vs[2], prm.d, wave_s, lane);
   // A bias that is the same for every query (query stride 0) is 64 values per key tile, the same for all lanes: wave 0
@@ -269,8 +320,13 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
       }
     }
     if (tile * kBwdTile + kBwdTile <= Sk && klo.ok && vlo.ok) {
-      copy_tile64_inside<T, D>(kbase, prm.ks[2], tile * kBwdTile, klo, smem + buf * TILE_BYTES, wave_s);
-      copy_tile64_inside<T, D>(vbase, prm.vs[2], tile * kBwdTile, vlo, smem + (2 + buf) * TILE_BYTES, wave_s);
+      if constexpr (ROOMY) {
+        copy_tile64_inside<T, D>(kbase, prm.ks[2], tile * kBwdTile, klo, smem + buf * TILE_BYTES, wave_s);
+        copy_tile64_inside<T, D>(vbase, prm.vs[2], tile * kBwdTile, vlo, smem + (2 + buf) * TILE_BYTES, wave_s);
+      } else {
+        copy_two_tiles64_inside<T, D>(kbase, prm.ks[2], klo, smem + buf * TILE_BYTES, vbase, prm.vs[2], vlo, smem + (2 + buf) * TILE_BYTES,
+                                      tile * kBwdTile, wave_s);
+      }
     } else {
       copy_tile64<T, D>(kbase, prm.ks[2], tile * kBwdTile, Sk, prm.d, smem + buf * TILE_BYTES, wave_s, lane);
       copy_tile64<T, D>(vbase, prm.vs[2], tile * kBwdTile, Sk, prm.d, smem + (2 + buf) * TILE_BYTES, wave_s, lane);
@@ -279,7 +335,8 @@ __global__ void __launch_bounds__(kBwdWaves * 64, 2) attn_bwd_dq_kernel(const At
   issue(0, 0);
   FO_LDS float* key_bias = (FO_LDS float*)(smem + 4 * TILE_BYTES);      // KBIAS: [2][64], bias / scale of the keys of a tile
   float key_bias_next = 0.0f;                                           // (wave 0) this lane's key of the tile after next
-  const float per_scale = KBIAS ? kLog2e / prm.scale_log2e : 0.0f;
+  // (wave-uniform, and told so: this kernel has no vector register to spare)
+  const float per_scale = KBIAS ? __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, kLog2e / prm.scale_log2e))) : 0.0f;
   const int64_t key_bias_row = KBIAS ? b * prm.bias.strides[0] + h * prm.bias.strides[1] : 0;
   if constexpr (KBIAS) {
     if (wave_s == 0) {
