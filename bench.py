@@ -80,22 +80,33 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def _settle(step, launches):
-    """`launches` untimed-for-the-result launches of `step` so that the clocks are where a sustained run has them; the
-    first and last per-launch times are reported to show what the phase did."""
+def _settle(step, launches, max_blocks=6, steady=0.015):
+    """Untimed-for-the-result launches of `step` so that the clocks are where a sustained run has them: blocks of
+    `launches`, repeated (at most `max_blocks` times) until the median launch time of a block is within `steady` of the
+    block before it - on some boxes the chip is still moving between a cold fast state and its sustained clock after one
+    block. The first and last per-launch times and the block medians are reported to show what the phase did."""
     import torch
 
     if launches <= 0:
         return {"launches": 0}
-    ev = _events(launches + 1)
-    ev[0].record()
-    for i in range(launches):
-        step()
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(launches)]
-    k = max(1, min(5, launches // 2))
-    return {"launches": launches, "ms_first": sum(ms[:k]) / k, "ms_last": sum(ms[-k:]) / k, "ms_max": max(ms)}
+    medians, first, ms_max = [], None, 0.0
+    while True:
+        ev = _events(launches + 1)
+        ev[0].record()
+        for i in range(launches):
+            step()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(launches)]
+        k = max(1, min(5, launches // 2))
+        if first is None:
+            first = sum(ms[:k]) / k
+        ms_max = max(ms_max, max(ms))
+        medians.append(sorted(ms)[launches // 2])
+        if len(medians) >= max_blocks or (len(medians) >= 2 and abs(medians[-1] - medians[-2]) <= steady * medians[-2]):
+            break
+    return {"launches": launches * len(medians), "ms_first": first, "ms_last": sum(ms[-k:]) / k, "ms_max": ms_max,
+            "block_medians_ms": [round(m, 5) for m in medians]}
 
 
 def _time_steps(step, steps, warmup, settle=0, before_each=None, wall_without_events=False):
@@ -140,6 +151,8 @@ def _time_steps(step, steps, warmup, settle=0, before_each=None, wall_without_ev
             gc.enable()
     per_launch = [starts[i].elapsed_time(ends[i]) for i in range(steps)]
     info = dict(info, kernel_ms_median=sorted(per_launch)[steps // 2])
+    if steps <= 64:
+        info["timed_launches_ms"] = [round(x, 4) for x in per_launch]   # (beside the settle blocks: shows a chip still changing clocks)
     return (wall_plain if wall_plain is not None else wall_ms / steps), sum(per_launch) / steps, min(per_launch), info
 
 
@@ -714,7 +727,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle", type=int, default=100,
-                    help="clock-settle launches ahead of the warm-up of every timed section (reported, not counted as warm-up)")
+                    help="clock-settle launches ahead of the warm-up of every timed section, in blocks of this many until two blocks in a row "
+                         "agree within 1.5 %% (at most six; reported, not counted as warm-up)")
     ap.add_argument("--path", choices=["both", "attn", "lion", "next", "copy", "clock", "power", "ablations"], default="both",
                     help="next: the reference's benchmark matrix (forward, backward, forward+backward with bias and dropout) and the "
                          "typed Lion kernels; copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
