@@ -80,16 +80,19 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def _settle(step, launches, max_blocks=6, steady=0.015):
+def _settle(step, launches, steady=0.015, min_seconds=1.0, max_seconds=4.0):
     """Untimed-for-the-result launches of `step` so that the clocks are where a sustained run has them: blocks of
-    `launches`, repeated (at most `max_blocks` times) until the median launch time of a block is within `steady` of the
-    block before it - on some boxes the chip is still moving between a cold fast state and its sustained clock after one
-    block. The first and last per-launch times and the block medians are reported to show what the phase did."""
+    `launches`, repeated until the phase has lasted `min_seconds` and the median launch time of a block is within `steady`
+    of the block before it (`max_seconds` at most). On some boxes of the pool the chip runs its first 0.2 s under
+    load fast, the next half second 15 % slower and settles in between after a second or two; a section that is timed
+    0.1 s after the load began measures that transient, not the run. The first and last per-launch times and the block
+    medians are reported to show what the phase did."""
     import torch
 
     if launches <= 0:
         return {"launches": 0}
     medians, first, ms_max = [], None, 0.0
+    t_begin = time.perf_counter()
     while True:
         ev = _events(launches + 1)
         ev[0].record()
@@ -103,32 +106,39 @@ def _settle(step, launches, max_blocks=6, steady=0.015):
             first = sum(ms[:k]) / k
         ms_max = max(ms_max, max(ms))
         medians.append(sorted(ms)[launches // 2])
-        if len(medians) >= max_blocks or (len(medians) >= 2 and abs(medians[-1] - medians[-2]) <= steady * medians[-2]):
+        elapsed = time.perf_counter() - t_begin
+        if elapsed >= max_seconds or (elapsed >= min_seconds and len(medians) >= 2 and abs(medians[-1] - medians[-2]) <= steady * medians[-2]):
             break
-    return {"launches": launches * len(medians), "ms_first": first, "ms_last": sum(ms[-k:]) / k, "ms_max": ms_max,
-            "block_medians_ms": [round(m, 5) for m in medians]}
+    shown = medians if len(medians) <= 12 else medians[:6] + medians[-6:]
+    return {"launches": launches * len(medians), "seconds": round(time.perf_counter() - t_begin, 3), "ms_first": first,
+            "ms_last": sum(ms[-k:]) / k, "ms_max": ms_max, "block_medians_ms": [round(m, 5) for m in shown]}
 
 
 def _time_steps(step, steps, warmup, settle=0, before_each=None, wall_without_events=False):
     """`settle` clock-settle launches, W untimed steps, then K timed steps bracketed by synchronize; per-launch durations
     from HIP events recorded on the stream the kernels are launched on (torch's current stream). `before_each(i)`, if
-    given, runs before timed step i outside its pair of events (fresh inputs for the step). With `wall_without_events`
-    the wall time per step comes from K further steps with no events between them (for kernels of a few tens of
-    microseconds, where the two event records per step are a sizeable part of a step)."""
+    given, runs before timed step i outside its pair of events (fresh inputs for the step; only then are the events
+    pairs). With `wall_without_events` the wall time per step comes from K further steps with no events between them
+    (for kernels of a few tens of microseconds, where the event records are a sizeable part of a step)."""
     import gc
 
     import torch
 
-    info = _settle(step, settle)
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    # (Python's cycle collector stays out of the timed steps: a full collection in this process takes tens of
-    # milliseconds of host time, which the events around a 30-microsecond launch see as the GPU waiting)
+    # Python's cycle collector stays out of the timed steps: a full collection in this process takes tens of
+    # milliseconds of host time, which the events around a 30-microsecond launch see as the GPU waiting. It runs before
+    # the settle phase, and the events are made there too, so that between the last warm-up step and the first timed one
+    # the chip is idle for no longer than the synchronize the contract asks for: on some boxes of the pool every pause
+    # under load is followed by some twenty launches that take up to 35 % longer.
     gc.collect()
     gc_was_on = gc.isenabled()
     gc.disable()
+    marks = _events(steps + 1)
+    starts, ends = (_events(steps), _events(steps)) if before_each is not None else (None, None)
     try:
+        info = _settle(step, settle)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
         wall_plain = None
         if wall_without_events:
             t0 = time.perf_counter()
@@ -136,20 +146,30 @@ def _time_steps(step, steps, warmup, settle=0, before_each=None, wall_without_ev
                 step()
             torch.cuda.synchronize()
             wall_plain = (time.perf_counter() - t0) * 1e3 / steps
-        starts, ends = _events(steps), _events(steps)
-        t0 = time.perf_counter()
-        for i in range(steps):
-            if before_each is not None:
+        if before_each is None:
+            # one event after every step (and one in front of the first): a launch's time runs from the end of the launch
+            # before it to its own end
+            t0 = time.perf_counter()
+            marks[0].record()
+            for i in range(steps):
+                step()
+                marks[i + 1].record()
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3
+            per_launch = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
+        else:
+            t0 = time.perf_counter()
+            for i in range(steps):
                 before_each(i)
-            starts[i].record()
-            step()
-            ends[i].record()
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3
+                starts[i].record()
+                step()
+                ends[i].record()
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3
+            per_launch = [starts[i].elapsed_time(ends[i]) for i in range(steps)]
     finally:
         if gc_was_on:
             gc.enable()
-    per_launch = [starts[i].elapsed_time(ends[i]) for i in range(steps)]
     info = dict(info, kernel_ms_median=sorted(per_launch)[steps // 2])
     if steps <= 64:
         info["timed_launches_ms"] = [round(x, 4) for x in per_launch]   # (beside the settle blocks: shows a chip still changing clocks)
@@ -728,7 +748,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--settle", type=int, default=100,
                     help="clock-settle launches ahead of the warm-up of every timed section, in blocks of this many until two blocks in a row "
-                         "agree within 1.5 %% (at most six; reported, not counted as warm-up)")
+                         "agree within 1.5 %% and a second has passed (reported, not counted as warm-up)")
     ap.add_argument("--path", choices=["both", "attn", "lion", "next", "copy", "clock", "power", "ablations"], default="both",
                     help="next: the reference's benchmark matrix (forward, backward, forward+backward with bias and dropout) and the "
                          "typed Lion kernels; copy: a plain 4 GiB device copy, the known-size reference that HBM byte counters are scaled by; "
