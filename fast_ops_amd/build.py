@@ -41,14 +41,30 @@ SOURCES = {
     "lion_typed.hip": ["-ffp-contract=off"],
     # attn_fwd.hip and attn_bwd.hip lay their inner loops out as fully unrolled micro-groups; the default size limit for
     # "#pragma unroll" would silently leave them rolled, with their register arrays in scratch memory.
+    # (attn_fwd.hip and attn_bwd.hip themselves are the C ABI and the kernel choice; their kernels are compiled as four
+    # units each, one per operand type and head_dim, which include them - in parallel, they are what takes the
+    # compiler's time)
     "attn_fwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_fwd_bf16_d64.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_fwd_bf16_d128.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_fwd_f16_d64.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_fwd_f16_d128.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
     "attn_bwd.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_bwd_bf16_d64.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_bwd_bf16_d128.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_bwd_f16_d64.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
+    "attn_bwd_f16_d128.hip": ["-mllvm", "-pragma-unroll-threshold=400000"],
     "dropout_mask.hip": [],
 }
+# sources that other sources include (a change in one of them makes every object stale, like a header's)
+INCLUDED_SOURCES = ["attn_fwd.hip", "attn_bwd.hip"]
 # sources whose generated assembly is checked by asm_lint: source -> regular expression of the kernel symbols to check
 # (the instantiations with a non-zero last template argument are timing experiments with wrong results by design)
 # (attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM>: DBG is the last but one)
-ASM_LINTED = {"attn_fwd.hip": r"attn_fwd_wide_kernel.*ELi0ELi\d+ELb[01]EEEvNS_10AttnParamsE", "attn_bwd.hip": r"attn_bwd_dkdv_pipe_kernel"}
+_PIPE = r"attn_bwd_dkdv_pipe_kernel"
+_WIDE = r"attn_fwd_wide_kernel.*ELi0ELi\d+ELb[01]EEEvNS_10AttnParamsE"
+ASM_LINTED = {"attn_fwd_bf16_d64.hip": _WIDE, "attn_fwd_bf16_d128.hip": _WIDE, "attn_fwd_f16_d64.hip": _WIDE, "attn_fwd_f16_d128.hip": _WIDE,
+              "attn_bwd_bf16_d64.hip": _PIPE, "attn_bwd_bf16_d128.hip": _PIPE, "attn_bwd_f16_d64.hip": _PIPE, "attn_bwd_f16_d128.hip": _PIPE}
 
 
 def _hipcc() -> str:
@@ -59,7 +75,7 @@ def _hipcc() -> str:
 
 
 def _newest_header_mtime() -> float:
-    paths = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))]
+    paths = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))] + [os.path.join(CSRC, f) for f in INCLUDED_SOURCES]
     paths.append(os.path.join(os.path.dirname(HERE), "include", "fastops.h"))
     return max(os.path.getmtime(p) for p in paths if os.path.exists(p))
 
@@ -140,7 +156,7 @@ def build_library(force: bool = False, verbose: bool = True, ablations: bool = F
         force = True
         with open(stamp, "w") as f:
             f.write(want)
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(lambda kv: _compile_one(hipcc, kv[0], kv[1], force, verbose), SOURCES.items()))
     need_link = force or not os.path.exists(LIB_PATH) or any(os.path.getmtime(o) > os.path.getmtime(LIB_PATH) for o in objs)
     if need_link:

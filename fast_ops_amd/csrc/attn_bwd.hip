@@ -1207,8 +1207,51 @@ static int launch_bwd(const AttnBwdParams& p, hipStream_t s) {
   return launch_status();
 }
 
+// every kernel of one operand type and head_dim behind one function, which one translation unit defines (see below)
+template <typename T, int D>
+int launch_bwd_of(const AttnBwdParams& p, bool causal, bool drop, bool has_bias, hipStream_t s) {
+  if (has_bias) {
+    if (drop) return causal ? launch_bwd<T, D, true, true, true>(p, s) : launch_bwd<T, D, false, true, true>(p, s);
+    return causal ? launch_bwd<T, D, true, false, true>(p, s) : launch_bwd<T, D, false, false, true>(p, s);
+  }
+  if (drop) return causal ? launch_bwd<T, D, true, true, false>(p, s) : launch_bwd<T, D, false, true, false>(p, s);
+  return causal ? launch_bwd<T, D, true, false, false>(p, s) : launch_bwd<T, D, false, false, false>(p, s);
+}
+// This file is compiled several times, in parallel: as it stands it is the C ABI and holds no kernel;
+// attn_bwd_bf16_d64.hip ... attn_bwd_f16_d128.hip include it with FO_ATTN_UNIT set and instantiate launch_bwd_of<T, D>.
+#ifndef FO_ATTN_UNIT
+#define FO_ATTN_UNIT 0
+#endif
+#define FO_ATTN_LAUNCH(UNIT, T, D) \
+  FO_ATTN_EXTERN_##UNIT template int launch_bwd_of<T, D>(const AttnBwdParams&, bool, bool, bool, hipStream_t);
+#if FO_ATTN_UNIT == 1
+#define FO_ATTN_EXTERN_1
+#else
+#define FO_ATTN_EXTERN_1 extern
+#endif
+#if FO_ATTN_UNIT == 2
+#define FO_ATTN_EXTERN_2
+#else
+#define FO_ATTN_EXTERN_2 extern
+#endif
+#if FO_ATTN_UNIT == 3
+#define FO_ATTN_EXTERN_3
+#else
+#define FO_ATTN_EXTERN_3 extern
+#endif
+#if FO_ATTN_UNIT == 4
+#define FO_ATTN_EXTERN_4
+#else
+#define FO_ATTN_EXTERN_4 extern
+#endif
+FO_ATTN_LAUNCH(1, __bf16, 64)
+FO_ATTN_LAUNCH(2, __bf16, 128)
+FO_ATTN_LAUNCH(3, _Float16, 64)
+FO_ATTN_LAUNCH(4, _Float16, 128)
+
 }  // namespace fo
 
+#if FO_ATTN_UNIT == 0
 using namespace fo;
 
 // ---- the same without a workspace argument and without any allocation: the workspace is a device array of this library.
@@ -1293,14 +1336,10 @@ static int attn_bwd_impl(const void* q, const void* k, const void* v, const void
                     (p.bias.strides[1] * elt) % 16 == 0 && (p.bias.strides[2] * elt) % 16 == 0;
     p.bias.vec_ok = bias && ((uintptr_t)bias % (4 * elt)) == 0 && p.bias.strides[0] % 4 == 0 && p.bias.strides[1] % 4 == 0 && p.bias.strides[2] % 4 == 0;
   }
-#define FO_BWD2(T, DD, BI) (drop ? (c ? launch_bwd<T, DD, true, true, BI>(p, s) : launch_bwd<T, DD, false, true, BI>(p, s)) \
-                                 : (c ? launch_bwd<T, DD, true, false, BI>(p, s) : launch_bwd<T, DD, false, false, BI>(p, s)))
-#define FO_BWD(T, DD) (bias ? FO_BWD2(T, DD, true) : FO_BWD2(T, DD, false))
   // kernels are compiled for 64 and 128 columns; a head_dim in between runs on the next one with zero columns
-  if (dtype == FO_DTYPE_BF16) return D > 64 ? FO_BWD(__bf16, 128) : FO_BWD(__bf16, 64);
-  return D > 64 ? FO_BWD(_Float16, 128) : FO_BWD(_Float16, 64);
-#undef FO_BWD
-#undef FO_BWD2
+  const bool has_bias = bias != nullptr;
+  if (dtype == FO_DTYPE_BF16) return D > 64 ? launch_bwd_of<__bf16, 128>(p, c, drop, has_bias, s) : launch_bwd_of<__bf16, 64>(p, c, drop, has_bias, s);
+  return D > 64 ? launch_bwd_of<_Float16, 128>(p, c, drop, has_bias, s) : launch_bwd_of<_Float16, 64>(p, c, drop, has_bias, s);
 }
 
 extern "C" int fo_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
@@ -1338,3 +1377,4 @@ extern "C" int fo_attn_bwd_ex(const void* q, const void* k, const void* v, const
                        extras->dropout_p, extras->dropout_seed, extras->dropout_offset, extras->bias, extras->bias_strides,
                        extras->bias_dtype, stream);
 }
+#endif  // FO_ATTN_UNIT == 0

@@ -1,0 +1,4 @@
+// The attention backward kernels for _Float16 operands at head_dim 128 as a translation unit of their own (attn_bwd.hip
+// says how the units divide the work; the build compiles them in parallel).
+#define FO_ATTN_UNIT 4
+#include "attn_bwd.hip"

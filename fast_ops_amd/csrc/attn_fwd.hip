@@ -30,6 +30,13 @@
 
 #include "attn_common.hpp"
 
+// This file is compiled several times, in parallel: as it stands it is the C ABI and the kernel choice, and holds no
+// kernel; attn_fwd_bf16_d64.hip ... attn_fwd_f16_d128.hip include it with FO_ATTN_UNIT set and instantiate launch<T, D>,
+// i.e. every kernel of one operand type and head_dim (the kernels are what takes the compiler's time).
+#ifndef FO_ATTN_UNIT
+#define FO_ATTN_UNIT 0
+#endif
+
 namespace fo {
 
 constexpr int kWaves = 4;
@@ -1201,7 +1208,7 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
 
 // heads per group in the causal order "heaviest query blocks of a group's heads first" of the kernels that take one
 // 128-row query block per workgroup (see launch_one)
-static int heavy_first_group(const AttnParams& p, int D) {
+[[maybe_unused]] static int heavy_first_group(const AttnParams& p, int D) {   // (used by the launchers only: not in every unit)
   const int64_t kv_bytes_head = (int64_t)p.Sk * D * 2 * 2, n_bh_x = ((int64_t)p.B * p.H) >> 3;
   const int order = tune(g_attn_order);
   int64_t group = order >= 0 ? order : 8 * n_bh_x * kv_bytes_head <= (256ll << 20) ? n_bh_x : (64ll << 20) / (8 * kv_bytes_head);
@@ -1364,7 +1371,7 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
 }
 
 template <typename T, int D>
-static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
+int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
   if (p.bias.ptr != nullptr) {
     // A bias that is the same for every query has kernels of its own: the pipelined ones where choose_kernel says so, else
     // the per-key form of the 128-row kernel, with or without dropout. (attn.variant 1 keeps the general bias kernel,
@@ -1430,8 +1437,37 @@ static int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t st
   return lazy ? launch_one<T, D, false, true, 0>(p, stream) : launch_one<T, D, false, false, 0>(p, stream);
 }
 
+// one translation unit per operand type and head_dim defines its launch<T, D>; the others see a declaration
+#define FO_ATTN_LAUNCH(UNIT, T, D)                                                                  \
+  FO_ATTN_EXTERN_##UNIT template int launch<T, D>(const AttnParams&, bool, bool, hipStream_t);
+#if FO_ATTN_UNIT == 1
+#define FO_ATTN_EXTERN_1
+#else
+#define FO_ATTN_EXTERN_1 extern
+#endif
+#if FO_ATTN_UNIT == 2
+#define FO_ATTN_EXTERN_2
+#else
+#define FO_ATTN_EXTERN_2 extern
+#endif
+#if FO_ATTN_UNIT == 3
+#define FO_ATTN_EXTERN_3
+#else
+#define FO_ATTN_EXTERN_3 extern
+#endif
+#if FO_ATTN_UNIT == 4
+#define FO_ATTN_EXTERN_4
+#else
+#define FO_ATTN_EXTERN_4 extern
+#endif
+FO_ATTN_LAUNCH(1, __bf16, 64)
+FO_ATTN_LAUNCH(2, __bf16, 128)
+FO_ATTN_LAUNCH(3, _Float16, 64)
+FO_ATTN_LAUNCH(4, _Float16, 128)
+
 }  // namespace fo
 
+#if FO_ATTN_UNIT == 0
 using namespace fo;
 
 // The checks on sizes and strides that fo_attn_fwd and fo_attn_fwd_kernel share, so that the query answers "rejected"
@@ -1544,3 +1580,4 @@ extern "C" int fo_attn_fwd_ex(const void* q, const void* k, const void* v, void*
   return attn_fwd_impl(q, k, v, o, lse, B, H, Sq, Sk, D, qs, ks, vs, os, softmax_scale, causal, dtype, extras->dropout_p,
                        extras->dropout_seed, extras->dropout_offset, extras->bias, extras->bias_strides, extras->bias_dtype, stream);
 }
+#endif  // FO_ATTN_UNIT == 0
