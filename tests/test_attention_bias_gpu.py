@@ -347,12 +347,13 @@ def test_per_key_bias_in_the_128_row_kernel_with_and_without_dropout(p_drop, D, 
     assert float(((o.float() - o1.float()).abs() - (2e-2 + 2e-2 * o1.float().abs())).max()) <= 0 and float((lse - lse1).abs().max()) <= 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
 @pytest.mark.parametrize("causal", [False, True])
-def test_per_key_bias_properties_at_the_headline_size(causal):
+def test_per_key_bias_properties_at_the_headline_size(causal, dtype):
     # B=2 H=16 S=8192 D=128 bf16 (the 256-row kernel with the bias row in LDS), by what the mathematics fixes: a bias that
     # is the same for every key changes nothing but LSE, which moves by that constant; -inf on the last keys is attention
     # over the keys before them; and the backward of both agrees with the backward without bias
-    B, H, S, D, dtype = 2, 16, 8192, 128, torch.bfloat16
+    B, H, S, D = 2, 16, 8192, 128
     assert _kernel_with_key_bias(B, H, S, S, D, causal) == 32
     g = torch.Generator().manual_seed(123)
     q, k, v, go = (torch.randn(B, H, S, D, generator=g).to(dtype).to(DEV) for _ in range(4))
