@@ -30,8 +30,8 @@ def _case(seed):
                 multi_query=r.random() < 0.2, bias=r.choice(BIAS_KINDS), bias_f32=r.random() < 0.5,
                 dropout=r.choice([0.0, 0.0, 0.1, 0.5]), scale=r.choice([None, None, 0.05, 0.3]),
                 # forward kernel (attn.variant): the library's choice, the 128-row kernel, the 256-row kernel with eight or
-                # four waves (drawn last, so that the other draws of a seed stay what they were; bias and dropout run on
-                # the 128-row kernel whatever is asked, head_dim 64 has no four-wave form)
+                # four waves (drawn last, so that the other draws of a seed stay what they were; dropout and a bias with a
+                # query stride run on the 128-row kernel whatever is asked, a per-key bias on the forms that exist for it)
                 variant=r.choice([-1, 0, 8, 8, 16, 16, 32, 32]))
 
 
