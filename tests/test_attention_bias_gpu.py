@@ -266,6 +266,16 @@ def test_per_key_bias_longer_than_the_pipelined_kernels_keep():
     # more than 8192 keys: the row of the bias no longer fits beside the tile rings, the plain kernel takes the call
     assert _kernel_with_key_bias(1, 12, 2048, 8256, 128, False) == 0
     assert _kernel_with_key_bias(1, 12, 2048, 8192, 128, False) in (8, 32)
+    B, H, Sq, Sk, D, dtype = 1, 12, 300, 8300, 128, torch.bfloat16
+    g = torch.Generator().manual_seed(8300)
+    q = torch.randn(B, H, Sq, D, generator=g).to(dtype)
+    k, v = (torch.randn(B, H, Sk, D, generator=g).to(dtype) for _ in range(2))
+    bias = torch.randn(B, 1, 1, Sk, generator=g) * 2.0
+    bias[..., 8200:8250] = float("-inf")
+    o, lse = attn_fwd_strided(q.to(DEV), k.to(DEV), v.to(DEV), (0, 1, 2, 3), False, None, None, bias.to(DEV))
+    o_ref, lse_ref = attention_fwd_oracle(q[:, :2], k[:, :2], v[:, :2], bias=bias)
+    err = (o[:, :2].float().cpu() - o_ref).abs()
+    assert float((err - (O_ATOL + O_RTOL * o_ref.abs())).max()) <= 0 and float((lse[:, :2].cpu() - lse_ref).abs().max()) <= LSE_ATOL
 
 
 # ---- backward with a bias that is the same for every query: the dQ kernel starts its score accumulators from it, the
