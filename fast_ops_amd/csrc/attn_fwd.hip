@@ -611,6 +611,7 @@ __host__ __device__ inline int wide_items(int n_qblk, bool causal) { return caus
 
 // keys of a per-key bias the pipelined kernel keeps in LDS (fp32, beside the rings: 128 + 32 of the 160 KiB at head_dim 128)
 constexpr int kVBiasKeys = 8192;
+constexpr float kNoKeyYet = -1.0e30f;   // reference of a row all of whose keys so far a bias of -inf has removed
 
 template <typename T, int D, bool CAUSAL, int QB, int DBG, int BM = kWideBM, bool VBIAS = false>
 __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 128 || VBIAS) ? 1 : 2) attn_fwd_wide_kernel(const AttnParams prm) {
@@ -620,8 +621,9 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // score in the base-2 domain and the running maximum, the lazily raised reference and LSE keep their meaning with
   // S + b / scale in the place of S. A step reads the 16 values of its 32 keys that a lane's registers hold (they
   // depend on the register and the half of the wave only) and adds them where the scores are scaled: one more VALU
-  // instruction per score. A bias of -inf removes a key; rows whose keys so far are all removed have the reference
-  // -inf, and every step of such a row takes the recovery path (left padding: a few steps per workgroup).
+  // instruction per score. A bias of -inf removes a key; a row whose keys so far are all removed has the reference
+  // kNoKeyYet, a large negative number, against which removed keys give 0 and the first key that counts overflows the
+  // row sum once (recovery path), which multiplies the row's empty O and l by 0 (left padding: one step per row).
   // BM = 256: the form described above. BM = 128 (QB = 1): the same pipeline with four waves x 32 rows, one query block
   // per workgroup in the 128-row kernel's order (heaviest causal blocks first), for shapes that give the chip too few
   // 256-row workgroups: a workgroup's time per key tile is what bounds those, and this pipeline's is less than half the
@@ -1014,10 +1016,9 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
 #pragma unroll
         for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, S[P][b2][r]);
         mloc = fmaxf(mloc, half_swap(mloc));
-        const float m_new = fmaxf(m_run[b2], mloc);                    // finite from the first sub-tile on: key 0 is never masked ...
-        const bool no_key_yet = VBIAS && m_new == -INFINITY;           // ... but a bias may have removed every key so far
-        const float alpha = no_key_yet ? 1.0f : __builtin_amdgcn_exp2f((m_run[b2] - m_new) * c);
-        const float mcn = no_key_yet ? 0.0f : m_new * c;
+        const float m_new = fmaxf(m_run[b2], mloc);                    // finite: key 0 is never masked (a bias: see kNoKeyYet)
+        const float alpha = __builtin_amdgcn_exp2f((m_run[b2] - m_new) * c);
+        const float mcn = m_new * c;
         float ps = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -1110,10 +1111,12 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
       mloc = fmaxf(mloc, (lim > -((r & 3) + 8 * (r >> 2))) ? -INFINITY : sv);
     }
     m_run[b2] = fmaxf(mloc, half_swap(mloc));
+    // (a bias may have removed every key of the sub-tile: the reference then starts from a large negative number
+    // instead of -inf, so that a removed key gives exp2(-inf) = 0 and not exp2(-inf + inf); the first key that counts
+    // overflows the row sum and the recovery path moves the reference to it, with O and l multiplied by exp2(-huge) = 0)
+    if constexpr (VBIAS) m_run[b2] = fmaxf(m_run[b2], kNoKeyYet);
   }
-  // (its reference is its own row maximum: every P <= 1 and no recovery - unless a bias removed all its keys)
-  if constexpr (VBIAS) step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1);
-  else step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1, N{});
+  step(0, P0{}, Y{}, N{}, Y{}, N{}, N{}, -1, N{});   // (its reference is its own row maximum: every P <= 1, no recovery)
   if (n_w > 1) step(1, P1{}, Y{}, Y{}, Y{}, N{}, N{}, -1); else step(1, P1{}, N{}, Y{}, Y{}, N{}, N{}, -1);
   // Should the steps above have parked registers in scratch memory (they do not at present), wait here, visibly to
   // the compiler, for any reload still in flight: otherwise it guards the first use inside the loops with a vmcnt(0)
