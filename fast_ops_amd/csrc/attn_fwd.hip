@@ -54,6 +54,7 @@ struct AttnParams {
   int n_qblk;
   int heavy_first;                      // 128-row kernel, causal: heads per group in the order of an XCD's workgroups, 0 = head by head (see launch_one)
   int order_n;                          // 128-row kernel, causal: entries of order_tab in use, 0 = none
+  int keep_on;                          // 256-row kernel, four waves: non-zero = copy the next query block's first tiles during the last tiles of a block
   uint8_t order_tab[kOrderTab];         // position in an XCD's launch order -> rank of the workgroup (0 = heaviest) that runs there
   DropoutParams drop;                   // used by the kernels instantiated with dropout only
   BiasParams bias;                      // used by the kernels instantiated with bias only
@@ -614,7 +615,8 @@ constexpr int kVBiasKeys = 8192;
 constexpr float kNoKeyYet = -1.0e30f;   // reference of a row all of whose keys so far a bias of -inf has removed
 
 template <typename T, int D, bool CAUSAL, int QB, int DBG, int BM = kWideBM, bool VBIAS = false>
-__global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 128 || VBIAS) ? 1 : 2) attn_fwd_wide_kernel(const AttnParams prm) {
+__global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 128 || VBIAS) ? 1 : 2) attn_fwd_wide_kernel(const AttnParams prm_arg) {
+  const AttnParams& prm = prm_arg;
   // VBIAS: an additive bias that is the same for every query of a head (query stride 0: the reference's "vector" bias,
   // flash_attention_triton.py:176-186, e.g. a key padding mask). The head's row of it, at most kVBiasKeys keys, is put
   // into LDS once per workgroup as fp32 divided by softmax_scale, so that (S + b / scale) * scale * log2 e is the biased
@@ -659,11 +661,16 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // A causal workgroup takes two query blocks, one after the other: block n-1-i (the heaviest left) and block i, so
   // that every workgroup has the same amount of work (n+1 tiles' worth) whatever i is. Non-causal: one block each.
   // (BM = 128: one block each, causal or not, heaviest blocks first as in attn_fwd_kernel.)
+  // KEEP_ON (four waves x 64 rows without bias): a workgroup may be given several work items, blockIdx.x, + gridDim.x,
+  // ... (the launcher decides: one item per workgroup, or one workgroup per CU that walks its share), and while it is
+  // in the last three tiles of a query block it already copies the first tiles of the next one - the second block of a
+  // causal pair, or the next item's - into the ring slots the tiles behind the end would have taken, and fetches that
+  // block's Q. The next block then starts without waiting for memory.
+  constexpr bool KEEP_ON = BM == kWideBM && QB == 2 && !VBIAS;
   const int n_bh = prm.B * prm.H;
   const int n_items = PAIRED ? wide_items(prm.n_qblk, true) : prm.n_qblk;
-  int bh, item;
-  {
-    const int id = blockIdx.x;
+  const int n_ids = n_items * n_bh;
+  auto decode = [&](int id, int& bh_, int& item_) {
     if ((n_bh & 7) == 0) {
       const int x = id & 7, j = id >> 3;          // XCD, position in that XCD's list
       if (BM != kWideBM && CAUSAL && prm.heavy_first > 0) {
@@ -671,26 +678,30 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
         const int n_bh_x = n_bh >> 3, per_group = prm.heavy_first * prm.n_qblk;
         const int grp = j / per_group, r = j - grp * per_group;
         const int heads = min(prm.heavy_first, n_bh_x - grp * prm.heavy_first);
-        bh = x + 8 * (grp * prm.heavy_first + r % heads);
-        item = r / heads;
+        bh_ = x + 8 * (grp * prm.heavy_first + r % heads);
+        item_ = r / heads;
       } else {
-        bh = x + 8 * (j / n_items);               // one head after the other
-        item = j % n_items;
+        bh_ = x + 8 * (j / n_items);               // one head after the other
+        item_ = j % n_items;
       }
     } else {
-      bh = id % n_bh;
-      item = id / n_bh;
+      bh_ = id % n_bh;
+      item_ = id / n_bh;
     }
-    if (BM != kWideBM && CAUSAL) item = prm.n_qblk - 1 - item;   // heaviest first
-  }
-  const int b = bh / prm.H, h = bh % prm.H;
-  const int n_pass = (PAIRED && prm.n_qblk - 1 - item != item) ? 2 : 1;
+    if (BM != kWideBM && CAUSAL) item_ = prm.n_qblk - 1 - item_;   // heaviest first
+  };
+  int wg_id = blockIdx.x;
+  int bh, item;
+  decode(wg_id, bh, item);
+  int pass = 0;
+  bool first_block = true, prefetched = false;
+  bool o_rows_whole = false;     // every row of the block before this one was stored (no store instruction may have been skipped)
   // Q^T fragments (B operand of S^T = K Q^T), QB blocks of 32 query rows, of the query block a pass works on. The
   // second pass's are fetched when the first pass has computed its last scores, so that they arrive while it
   // normalises and writes its O.
   i32x4 qf[QB][KSTEPS];
-  auto load_q = [&](int for_qblk) {
-    const T* qb_base = (const T*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  auto load_q = [&](int of_bh, int for_qblk) {
+    const T* qb_base = (const T*)prm.q + (of_bh / prm.H) * prm.qs[0] + (of_bh % prm.H) * prm.qs[1];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const int qrow = min(for_qblk * BM + wave_s * 32 * QB + 32 * qb + l32, prm.Sq - 1);
@@ -701,16 +712,38 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   };
   FO_LDS float* vbias = (FO_LDS float*)(smem + 2 * kRing * TILE_BYTES) + 4 * hh;   // (this lane's half: its registers' keys start 4 further)
   if constexpr (VBIAS) {
-    const int64_t brow = b * prm.bias.strides[0] + h * prm.bias.strides[1];
+    const int64_t brow = (bh / prm.H) * prm.bias.strides[0] + (bh % prm.H) * prm.bias.strides[1];
     const float per_scale = 1.4426950408889634f / prm.scale_log2e;
     const int n_pad = (prm.Sk + kBN - 1) / kBN * kBN;                  // at most kVBiasKeys: the launcher checks
     for (int i = tid; i < n_pad; i += kWideWaves * 64)
       ((FO_LDS float*)(smem + 2 * kRing * TILE_BYTES))[i] = load_bias<T>(prm.bias, brow + min(i, prm.Sk - 1)) * per_scale;
     __syncthreads();
   }
-  for (int pass = 0; pass < n_pass; ++pass) {
+  for (;;) {   // query blocks of this workgroup
+#if defined(__HIP_DEVICE_COMPILE__)
+  // (KEEP_ON: the kernel's arguments are read afresh for every block, through a copy of their address that the compiler
+  // cannot see through. Otherwise everything derived from them is kept across the loop - far more than there are scalar
+  // registers - and the moves to and from the lanes of spare vector registers cost a block about a microsecond.)
+  typedef const __attribute__((address_space(4))) AttnParams* ArgPtr;
+  ArgPtr args_here = (ArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
+  if constexpr (KEEP_ON) asm volatile("" : "+s"(args_here));
+  decltype(auto) prm = [&]() -> decltype(auto) { if constexpr (KEEP_ON) return (*args_here); else return (prm_arg); }();
+#else
+  const AttnParams& prm = prm_arg;
+#endif
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int n_pass = (PAIRED && prm.n_qblk - 1 - item != item) ? 2 : 1;
   const int qblk = PAIRED ? (pass == 0 ? prm.n_qblk - 1 - item : item) : item;
-  if (pass > 0) {
+  // the block after this one
+  bool has_next = false;
+  int next_bh = bh, next_item = item, next_qblk = item;       // (second pass of a pair: block `item` of the same head)
+  if (pass + 1 < n_pass) has_next = true;
+  else if (KEEP_ON && wg_id + (int)gridDim.x < n_ids) {
+    decode(wg_id + (int)gridDim.x, next_bh, next_item);
+    next_qblk = PAIRED ? prm.n_qblk - 1 - next_item : next_item;
+    has_next = true;
+  }
+  if (!first_block && !prefetched) {
     // the other waves may still be reading the rings, and this wave's stores of O still count as memory operations in flight
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -755,9 +788,8 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // batch t is this wave's to issue
   auto my_turn = [&](int t) -> bool { return ISSUERS == 1 || ((t + 4) & 1) == (wave_s >> 2); };
   // one tile of K (ring 0) or V (ring 1) into slot tile % kRing
-  auto issue = [&](auto is_v, int tile) {
+  auto issue = [&](auto is_v, int tile, const T* base) {
     constexpr bool V = decltype(is_v)::value;
-    const T* base = V ? vbase : kbase;
     const int64_t stride = V ? prm.vs[2] : prm.ks[2];
     const int key0 = tile * kBN;
     FO_LDS char* dst = smem + (kRing * (V ? 1 : 0) + (tile & (kRing - 1))) * TILE_BYTES;
@@ -810,15 +842,36 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
       return 2 * NBLK;
     }
     int n = 0;
-    if (t + 3 < n_tiles && t + 3 >= 0) { issue(std::false_type{}, t + 3); n += NBLK; }
-    if (t + 2 < n_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2); n += NBLK; }
+    if (t + 3 < n_tiles && t + 3 >= 0) { issue(std::false_type{}, t + 3, kbase); n += NBLK; }
+    if (t + 2 < n_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2, vbase); n += NBLK; }
     return n;
   };
-  issue_batch(-3);
-  issue_batch(-2);
-  int last_batch = issue_batch(-1);
+  // The first three batches of the NEXT block (t = -3, -2, -1: K(0) | K(1), V(0) | K(2), V(1)), issued at the tops of
+  // this block's last three tiles. Its tile i goes to ring slot i % kRing, which is the slot this block's tile
+  // n_tiles + i would have taken when n_tiles is a multiple of kRing - only then is there a prefetch.
+  int next_tiles = 0;
+  const T* next_kbase = kbase;
+  const T* next_vbase = vbase;
+  if (has_next) {
+    next_tiles = CAUSAL ? (min(Sk, next_qblk * BM + BM) + kBN - 1) / kBN : n_tiles;
+    next_kbase = (const T*)prm.k + (next_bh / prm.H) * prm.ks[0] + (next_bh % prm.H) * prm.ks[1];
+    next_vbase = (const T*)prm.v + (next_bh / prm.H) * prm.vs[0] + (next_bh % prm.H) * prm.vs[1];
+  }
+  const bool prefetch_next = KEEP_ON && has_next && n_tiles >= kRing && (n_tiles & (kRing - 1)) == 0 && prm.keep_on != 0;
+  auto issue_batch_next = [&](int t) -> int {
+    int n = 0;
+    if (t + 3 < next_tiles) { issue(std::false_type{}, t + 3, next_kbase); n += NBLK; }
+    if (t + 2 < next_tiles && t + 2 >= 0) { issue(std::true_type{}, t + 2, next_vbase); n += NBLK; }
+    return n;
+  };
+  int last_batch = 0;
+  if (!prefetched) {
+    issue_batch(-3);
+    issue_batch(-2);
+    last_batch = issue_batch(-1);
+  }
 
-  if (pass == 0) load_q(qblk);
+  if (first_block) load_q(bh, qblk);
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
@@ -1063,6 +1116,9 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
     if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
     if (spread_this) { last_batch = 2 * DMA_PER_WAVE; return true; }   // the steps of this tile issue them
     last_batch = (DBG & 1) ? 0 : issue_batch(j);
+    if constexpr (KEEP_ON) {
+      if (prefetch_next && j >= n_tiles - 3) last_batch += issue_batch_next(j - n_tiles);
+    }
     return false;
   };
   // Tiles that need the mask (causal diagonal, keys past the end) are a suffix of the wave's tiles. The hot loops are
@@ -1077,7 +1133,11 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // every reload is waited for with a vmcnt wait that also covers the copies in flight. So all three batches issued
   // above land before it starts - K(0), K(1) and V(0) have to anyway - and batch 0, K(3) and V(2) into slots nobody
   // has used yet, goes out after it, in front of the loops.)
-  if (!(DBG & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // (A block whose tiles were copied ahead: its copies and its Q loads were issued before the stores of the previous
+  // block's O, and memory operations complete in order - the last stores of O, one 32-row block's worth, may stay in
+  // flight. They are counted, so only where none of them can have been skipped.)
+  if (KEEP_ON && prefetched && o_rows_whole) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(32 * (ROW_BYTES / 16) / 64) : "memory");
+  else if (!(DBG & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (!(DBG & 64)) __builtin_amdgcn_s_barrier();
   {
     const uint32_t kb0 = k_lane + sub_base(0), kb1 = k_lane + sub_base(1);
@@ -1162,7 +1222,7 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // tiles in which this wave has nothing to do (causal): keep feeding the workgroup's rings
   for (; j < n_tiles; ++j) tile_top(j);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (PAIRED && pass + 1 < n_pass) load_q(item);   // (the second pass works on query block `item`)
+  if (has_next) load_q(next_bh, next_qblk);   // (they arrive while this block's O is written)
 
   // ---- epilogue: normalise, write O and LSE
 #pragma unroll
@@ -1171,14 +1231,29 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // 8 bytes per lane, 16 per row and instruction. Instead the wave's rows are staged in LDS (the rings are free once
   // every wave is past its last tile; rows padded by 16 bytes against bank conflicts) and leave as whole 16-byte
   // pieces, 64 lanes covering four consecutive 256-byte rows per instruction.
+  // (KEEP_ON: the first ring slots may already hold the next block's tiles. The rows are staged one 32-row block at a
+  // time behind them, from the third slot of the V ring on - free once every wave is past its last tile - into the
+  // 32 KiB after the rings.)
   __syncthreads();
+  constexpr int CH = ROW_BYTES / 16;                    // 16-byte pieces per row
   constexpr int OROW = ROW_BYTES + 16;
-  FO_LDS char* stage = smem + wave_s * (32 * QB) * OROW;
+  constexpr int STAGE_ROWS = KEEP_ON ? 32 : 32 * QB;    // rows a wave stages at a time
+  FO_LDS char* stage = smem + (KEEP_ON ? (kRing + 2) * TILE_BYTES : 0) + wave_s * STAGE_ROWS * OROW;
+  T* obase = (T*)prm.o + b * prm.os[0] + h * prm.os[1];
+  auto write_rows = [&](int first_row, int rows) {      // staged rows [0, rows) are query rows q0w + first_row ..
+#pragma unroll
+    for (int it = 0; it < STAGE_ROWS * CH / 64; ++it) {
+      const int idx = it * 64 + lane, row = idx / CH, ch = idx % CH;
+      const i32x4 piece = *(FO_LDS const i32x4*)(stage + row * OROW + ch * 16);
+      if (row < rows && q0w + first_row + row < Sq) *(i32x4*)(obase + (int64_t)(q0w + first_row + row) * prm.os[2] + ch * 8) = piece;
+    }
+  };
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = l_run[qb] + half_swap(l_run[qb]);
     const float inv = 1.0f / l_tot;
     const int qi = q0w + 32 * qb + l32;
+    const int srow = KEEP_ON ? l32 : 32 * qb + l32;
 #pragma unroll
     for (int db = 0; db < DBLK; ++db) {
       f32x16 t = oacc[db][qb];
@@ -1189,24 +1264,24 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
         vec4 o4;
 #pragma unroll
         for (int u = 0; u < 4; ++u) o4[u] = (T)(t[rg * 4 + u] * inv);
-        *(FO_LDS vec4*)(stage + (32 * qb + l32) * OROW + (32 * db + 8 * rg + 4 * hh) * 2) = o4;
+        *(FO_LDS vec4*)(stage + srow * OROW + (32 * db + 8 * rg + 4 * hh) * 2) = o4;
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     if (qi < Sq && prm.lse != nullptr && hh == 0)
       prm.lse[(int64_t)bh * Sq + qi] = (m_run[qb] * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+    if constexpr (KEEP_ON) write_rows(32 * qb, 32);
   }
-  {
-    constexpr int CH = ROW_BYTES / 16;                  // 16-byte pieces per row
-    T* obase = (T*)prm.o + b * prm.os[0] + h * prm.os[1];
-#pragma unroll
-    for (int it = 0; it < 32 * QB * CH / 64; ++it) {
-      const int idx = it * 64 + lane, row = idx / CH, ch = idx % CH;
-      const i32x4 piece = *(FO_LDS const i32x4*)(stage + row * OROW + ch * 16);
-      if (q0w + row < Sq) *(i32x4*)(obase + (int64_t)(q0w + row) * prm.os[2] + ch * 8) = piece;
-    }
-  }
-  }   // pass
+  if constexpr (!KEEP_ON) write_rows(0, 32 * QB);
+
+  // ---- on to the next block, if there is one
+  if (!has_next) break;
+  prefetched = prefetch_next;
+  o_rows_whole = q0w + 32 * QB <= Sq;
+  first_block = false;
+  if (pass + 1 < n_pass) ++pass;
+  else { wg_id += (int)gridDim.x; bh = next_bh; item = next_item; pass = 0; }
+  }   // query blocks
 }
 
 // heads per group in the causal order "heaviest query blocks of a group's heads first" of the kernels that take one
@@ -1236,10 +1311,22 @@ static int device_cus() {
 
 template <typename T, int D, bool CAUSAL, int QB, int DBG = 0, int BM = kWideBM, bool VBIAS = false>
 static int launch_wide(AttnParams p, hipStream_t stream) {
-  const size_t lds = 2 * (size_t)kRing * kBN * D * 2 + (VBIAS ? kVBiasKeys * 4 : 0);
+  constexpr bool KEEP_ON = BM == kWideBM && QB == 2 && !VBIAS;      // (as in the kernel)
+  // rings; bias row; or the rows of O staged behind the first six slots of the rings, 32 rows of D + 8 elements per wave
+  const size_t lds = KEEP_ON ? (size_t)(kRing + 2) * kBN * D * 2 + 4 * 32 * (D * 2 + 16) : 2 * (size_t)kRing * kBN * D * 2 + (VBIAS ? kVBiasKeys * 4 : 0);
   if (VBIAS && (p.Sk + kBN - 1) / kBN * kBN > kVBiasKeys) return FO_ERR_UNSUPPORTED;
   p.n_qblk = (p.Sq + BM - 1) / BM;
-  const unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);
+  unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);
+  p.keep_on = 0;
+  if (KEEP_ON) {
+    // attn.keep_on: 0 = one work item per workgroup and no copies ahead for the next query block; 1 = copies ahead for
+    // the second block of a causal pair; 2 (default) = also one workgroup per CU that walks its share of the items
+    // (blockIdx.x, + gridDim.x, ...: a multiple of 8 apart, so that an XCD keeps its heads)
+    const int mode = tune(g_attn_keep_on) < 0 ? 2 : tune(g_attn_keep_on);
+    p.keep_on = mode != 0;
+    const unsigned wgs = (unsigned)(device_cus() / 8 * 8);
+    if (mode == 2 && wgs >= 8 && grid > wgs) grid = wgs;
+  }
   p.heavy_first = (CAUSAL && BM != kWideBM) ? heavy_first_group(p, D) : 0;
   p.order_n = 0;
   static const hipError_t attr = hipFuncSetAttribute((const void*)attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM, VBIAS>,

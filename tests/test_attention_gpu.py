@@ -221,6 +221,47 @@ def test_ragged_and_unequal_lengths(shape, causal, D, kernel_variant):
     _run_and_check(B, H, Sq, Sk, D, torch.bfloat16, causal, seed=Sq * 1000 + Sk)
 
 
+# (B, H, Sq, Sk, D, causal): more work items than the chip has CUs, so that with attn.keep_on 2 (the default) a workgroup of
+# the four-wave 256-row kernel walks several of them and copies the next block's first tiles during a block's last ones
+# (key counts that are a multiple of 256) or falls back to waiting (the others); heads in and out of the XCD dealing
+# (multiples of 8 or not); a ragged last key tile; fewer key tiles than the three copied ahead; Sq above Sk when causal.
+WALKED = [(4, 40, 1024, 1024, 128, False), (4, 40, 1000, 1000, 128, True), (3, 37, 900, 700, 64, False), (5, 24, 1536, 100, 128, False),
+          (2, 64, 2048, 2048, 64, True), (2, 72, 2048, 512, 128, True), (3, 24, 1280, 1280, 128, True), (2, 40, 1792, 1000, 64, False)]
+
+
+@pytest.mark.parametrize("shape", WALKED)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+def test_work_items_walked_by_one_workgroup_per_cu(shape, dtype):
+    B, H, Sq, Sk, D, causal = shape
+    q, k, v = _qkv(B, H, Sq, Sk, D, dtype, seed=Sq + Sk)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    got = {}
+    _lib.tune_set("attn.variant", _lib.FO_ATTN_KERNEL_ROWS256_W4)
+    try:
+        assert _kernel_taken(qd, kd, vd, causal) == _lib.FO_ATTN_KERNEL_ROWS256_W4
+        for mode in (0, 1, 2, -1):
+            _lib.tune_set("attn.keep_on", mode)
+            # (the allocator hands the blocks freed last to the next request of their size: the outputs start as NaN, and
+            # a block that nobody worked on would show)
+            o = lse = None
+            junk = (torch.full_like(qd, float("nan")), torch.full((B, H, Sq), float("nan"), device=DEV))
+            del junk
+            o, lse = multi_head_attention(qd, kd, vd, causal=causal, return_lse=True)
+            torch.cuda.synchronize()
+            got[mode] = (o.cpu(), lse.cpu())
+            assert torch.isfinite(got[mode][0].float()).all() and torch.isfinite(got[mode][1]).all(), f"attn.keep_on {mode}"
+    finally:
+        _lib.tune_set("attn.keep_on", -1)
+        _lib.tune_set("attn.variant", -1)
+    # the same arithmetic in the same order whoever walks the items: identical bits
+    for mode in (1, 2, -1):
+        assert torch.equal(got[0][0], got[mode][0]) and torch.equal(got[0][1], got[mode][1]), f"attn.keep_on {mode} differs from 0"
+    o, lse = got[2]
+    for b, h in [(0, 0), (B - 1, H - 1), (B // 2, H // 3), (B - 1, 7)]:
+        o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], causal=causal)
+        _check(o[b:b + 1, h:h + 1], lse[b:b + 1, h:h + 1], o_ref, lse_ref, f"{shape} {dtype} slice ({b},{h})")
+
+
 @pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)

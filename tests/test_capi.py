@@ -151,7 +151,7 @@ def test_tune_hook():
     assert lib.fo_tune_set(b"lion.variant", -1) == 0
     assert lib.fo_tune_set(b"no.such.key", 1) == -8
     # every key the kernels read: default -1 (the library's choice), settable, readable
-    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn.balance", 0), (b"attn_bwd.order", 2)):
+    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn.balance", 0), (b"attn.keep_on", 1), (b"attn_bwd.order", 2)):
         assert lib.fo_tune_get(key) == -1
         assert lib.fo_tune_set(key, value) == 0 and lib.fo_tune_get(key) == value
         assert lib.fo_tune_set(key, -1) == 0 and lib.fo_tune_get(key) == -1
@@ -168,6 +168,7 @@ def test_tune_hook_accepts_only_kernels_that_compute_the_function():
         assert lib.fo_tune_get(b"attn.variant") == 32          # a refused value changes nothing
     assert lib.fo_tune_set(b"attn.variant", -1) == 0
     assert lib.fo_tune_set(b"attn_bwd.variant", 2) == -8
+    assert lib.fo_tune_set(b"attn.keep_on", 3) == -8
     assert lib.fo_tune_set(b"lion.variant", 32) == -8
 
 
