@@ -724,6 +724,7 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // (KEEP_ON: the kernel's arguments are read afresh for every block, through a copy of their address that the compiler
   // cannot see through. Otherwise everything derived from them is kept across the loop - far more than there are scalar
   // registers - and the moves to and from the lanes of spare vector registers cost a block about a microsecond.)
+  // (prm_arg is the kernel's only argument: it sits at the start of the argument segment)
   typedef const __attribute__((address_space(4))) AttnParams* ArgPtr;
   ArgPtr args_here = (ArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
   if constexpr (KEEP_ON) asm volatile("" : "+s"(args_here));
@@ -1322,7 +1323,8 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
     // attn.keep_on: 0 = one work item per workgroup and no copies ahead for the next query block; 1 = copies ahead for
     // the second block of a causal pair; 2 (default) = also one workgroup per CU that walks its share of the items
     // (blockIdx.x, + gridDim.x, ...: a multiple of 8 apart, so that an XCD keeps its heads)
-    const int mode = tune(g_attn_keep_on) < 0 ? 2 : tune(g_attn_keep_on);
+    const int asked = tune(g_attn_keep_on);
+    const int mode = asked < 0 ? 2 : asked;
     p.keep_on = mode != 0;
     const unsigned wgs = (unsigned)(device_cus() / 8 * 8);
     if (mode == 2 && wgs >= 8 && grid > wgs) grid = wgs;
