@@ -1431,7 +1431,9 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // 28 % less time). Four-wave form against the 128-row kernel: non-causal 1024 keys +2 %, 2048 -3 %, 4096 -6 %,
     // 8192 -6.5 %, 16384 -6 %; causal 2048 +3 %, 4096 -2 %, 8192 -5 %, 16384 -8 %. (The eight-wave form is 4-5 % behind
     // the four-wave form everywhere: non-causal 1024 keys +20 %, 4096 +0.6 %, 16384 -1.8 % against the 128-row kernel.)
-    if (D == 64 && keys < (causal ? 8192 : 4096)) wide = false;
+    // Since the four-wave form's workgroups walk their items, without bias: non-causal 1024 keys +6 %, 2048 +2 %, 3072
+    // -0.8 %, 4096 -1 %; causal 2048 +2 %, 4096 -8 %, 6144 -4.5 %, 8192 -6.5 %.
+    if (D == 64 && keys < (causal && !key_bias ? 4096 : causal ? 8192 : 4096)) wide = false;
     v = wide ? FO_ATTN_KERNEL_ROWS256_W8 : FO_ATTN_KERNEL_ROWS128;
     // Few workgroups for the chip (12 heads of a tensor-parallel split, short batches): what bounds the launch then is
     // the time a workgroup takes per key tile, not throughput, and 128-row workgroups in the pipelined kernel take less
@@ -1449,8 +1451,10 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // MFMAs, which costs less energy (at full load the chip's clock is what its power budget leaves) but more cycles per
     // tile, and its longer pipeline fill and drain have to be spread over enough tiles. Measured on one box, new form
     // against the eight-wave form: non-causal 2048 keys -1.0 %, 4096 -2.3 %, 8192 -2.5 %; causal 3072 +3 %, 4096 +1 %,
-    // 8192 -0.7 %, 16384 -1.8 %.
-    if (v == FO_ATTN_KERNEL_ROWS256_W8 && (D == 64 || keys >= (causal ? 6144 : 2048))) v = FO_ATTN_KERNEL_ROWS256_W4;
+    // 8192 -0.7 %, 16384 -1.8 %. With its workgroups walking their items (attn.keep_on), on one box: non-causal 512 keys
+    // -4 %, 768 -2 %, 1024 -2.5 %, 1536 -1 %, 2048 -1.5 %; causal 2048 +3.5 %, 3072 +2 %, 4096 +1.7 %, 6144 +2.4 %,
+    // 8192 -1 to -3 % (a causal block's diagonal costs the 64-row waves more than the 32-row ones).
+    if (v == FO_ATTN_KERNEL_ROWS256_W8 && (D == 64 || keys >= (causal ? 8192 : 512))) v = FO_ATTN_KERNEL_ROWS256_W4;
   }
   if (v >= 256) return v;
   if (!wide_ok && v >= FO_ATTN_KERNEL_ROWS128_PIPE) v = FO_ATTN_KERNEL_ROWS128;

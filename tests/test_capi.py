@@ -205,13 +205,15 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
         assert k(2, 16, 8192, 8192, 128, 1) == W4            # the headline shape: 512 workgroups of two query blocks
         assert k(16, 32, 2048, 2048, 128, 0) == W4           # B=16 H=32 S=2048 non-causal
         assert k(8, 12, 1024, 1024, 64, 1) == R128           # the GPT-2-small shape
-        assert k(2, 16, 4096, 4096, 128, 1) == W8            # fewer than 6144 keys, causal: eight waves
+        assert k(2, 16, 4096, 4096, 128, 1) == W8 and k(4, 16, 6144, 6144, 128, 1) == W8   # fewer than 8192 keys, causal: eight waves
         assert k(8, 16, 1024, 1024, 128, 1) == W8            # causal from 1024 queries on: 256 workgroups, one round
         assert k(12, 16, 1024, 1024, 128, 1) == R128         # 384 workgroups would leave half of the second round empty
         assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
-        assert k(16, 16, 512, 512, 128, 0) == W8 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups
+        assert k(16, 16, 512, 512, 128, 0) == W4 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups; non-causal: four waves
+        assert k(32, 16, 256, 256, 128, 0) == W8             # (below 512 keys the eight-wave form stays)
         assert k(1, 8, 8192, 8192, 64, 0) == W4 and k(4, 8, 4096, 4096, 64, 0) == W4 and k(8, 8, 2048, 2048, 64, 0) == R128   # head_dim 64: long rows only,
-        assert k(1, 8, 16384, 16384, 64, 1) == W4 and k(2, 16, 8192, 8192, 64, 1) == W4 and k(4, 16, 4096, 4096, 64, 1) == R128  # and four waves
+        assert k(1, 8, 16384, 16384, 64, 1) == W4 and k(2, 16, 8192, 8192, 64, 1) == W4 and k(4, 16, 4096, 4096, 64, 1) == W4  # and four waves
+        assert k(8, 16, 2048, 2048, 64, 1) == R128 and k(4, 16, 4096, 4096, 64, 1, bias=2) == R128   # (causal from 4096 keys, with a per-key bias from 8192)
         # too few workgroups for the chip (12 heads of a tensor-parallel split): 128-row workgroups in the pipelined kernel
         assert k(1, 12, 2048, 2048, 128, 1) == PIPE and k(1, 12, 2048, 2048, 128, 0) == PIPE and k(1, 12, 4096, 4096, 128, 1) == PIPE
         # long rows of keys at head_dim 128: the 256-row kernel already with three quarters of one round of workgroups
