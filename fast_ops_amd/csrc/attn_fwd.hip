@@ -54,7 +54,7 @@ struct AttnParams {
   int n_qblk;
   int heavy_first;                      // 128-row kernel, causal: heads per group in the order of an XCD's workgroups, 0 = head by head (see launch_one)
   int order_n;                          // 128-row kernel, causal: entries of order_tab in use, 0 = none
-  int keep_on;                          // 256-row kernel, four waves: non-zero = copy the next query block's first tiles during the last tiles of a block
+  int keep_on;                          // 256-row kernel without bias: non-zero = copy the next query block's first tiles during the last tiles of a block
   uint8_t order_tab[kOrderTab];         // position in an XCD's launch order -> rank of the workgroup (0 = heaviest) that runs there
   DropoutParams drop;                   // used by the kernels instantiated with dropout only
   BiasParams bias;                      // used by the kernels instantiated with bias only
@@ -661,12 +661,12 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // A causal workgroup takes two query blocks, one after the other: block n-1-i (the heaviest left) and block i, so
   // that every workgroup has the same amount of work (n+1 tiles' worth) whatever i is. Non-causal: one block each.
   // (BM = 128: one block each, causal or not, heaviest blocks first as in attn_fwd_kernel.)
-  // KEEP_ON (four waves x 64 rows without bias): a workgroup may be given several work items, blockIdx.x, + gridDim.x,
+  // KEEP_ON (256 rows without bias): a workgroup may be given several work items, blockIdx.x, + gridDim.x,
   // ... (the launcher decides: one item per workgroup, or one workgroup per CU that walks its share), and while it is
   // in the last three tiles of a query block it already copies the first tiles of the next one - the second block of a
   // causal pair, or the next item's - into the ring slots the tiles behind the end would have taken, and fetches that
   // block's Q. The next block then starts without waiting for memory.
-  constexpr bool KEEP_ON = BM == kWideBM && QB == 2 && !VBIAS;
+  constexpr bool KEEP_ON = BM == kWideBM && !VBIAS;
   const int n_bh = prm.B * prm.H;
   const int n_items = PAIRED ? wide_items(prm.n_qblk, true) : prm.n_qblk;
   const int n_ids = n_items * n_bh;
@@ -1239,7 +1239,11 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   constexpr int CH = ROW_BYTES / 16;                    // 16-byte pieces per row
   constexpr int OROW = ROW_BYTES + 16;
   constexpr int STAGE_ROWS = KEEP_ON ? 32 : 32 * QB;    // rows a wave stages at a time
-  FO_LDS char* stage = smem + (KEEP_ON ? (kRing + 2) * TILE_BYTES : 0) + wave_s * STAGE_ROWS * OROW;
+  // (eight waves at head_dim 128: seven of them fit there, the first one stages in the last slot of the K ring)
+  constexpr bool STAGE_SPLIT = KEEP_ON && (kRing + 2) * TILE_BYTES + kWideWaves * STAGE_ROWS * OROW > 160 * 1024;
+  FO_LDS char* stage = !KEEP_ON ? smem + wave_s * STAGE_ROWS * OROW
+                     : (STAGE_SPLIT && wave_s == 0) ? smem + (kRing - 1) * TILE_BYTES
+                     : smem + (kRing + 2) * TILE_BYTES + (wave_s - (STAGE_SPLIT ? 1 : 0)) * STAGE_ROWS * OROW;
   T* obase = (T*)prm.o + b * prm.os[0] + h * prm.os[1];
   auto write_rows = [&](int first_row, int rows) {      // staged rows [0, rows) are query rows q0w + first_row ..
 #pragma unroll
@@ -1312,9 +1316,12 @@ static int device_cus() {
 
 template <typename T, int D, bool CAUSAL, int QB, int DBG = 0, int BM = kWideBM, bool VBIAS = false>
 static int launch_wide(AttnParams p, hipStream_t stream) {
-  constexpr bool KEEP_ON = BM == kWideBM && QB == 2 && !VBIAS;      // (as in the kernel)
+  constexpr bool KEEP_ON = BM == kWideBM && !VBIAS;      // (as in the kernel)
   // rings; bias row; or the rows of O staged behind the first six slots of the rings, 32 rows of D + 8 elements per wave
-  const size_t lds = KEEP_ON ? (size_t)(kRing + 2) * kBN * D * 2 + 4 * 32 * (D * 2 + 16) : 2 * (size_t)kRing * kBN * D * 2 + (VBIAS ? kVBiasKeys * 4 : 0);
+  // (eight waves at head_dim 128: seven of them there, see the kernel)
+  constexpr int kWavesHere = BM / (32 * QB);
+  constexpr size_t kStageAll = (size_t)(kRing + 2) * kBN * D * 2 + kWavesHere * 32 * (D * 2 + 16);
+  const size_t lds = KEEP_ON ? (kStageAll > 160 * 1024 ? kStageAll - 32 * (D * 2 + 16) : kStageAll) : 2 * (size_t)kRing * kBN * D * 2 + (VBIAS ? kVBiasKeys * 4 : 0);
   if (VBIAS && (p.Sk + kBN - 1) / kBN * kBN > kVBiasKeys) return FO_ERR_UNSUPPORTED;
   p.n_qblk = (p.Sq + BM - 1) / BM;
   unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);

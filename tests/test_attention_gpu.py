@@ -222,7 +222,7 @@ def test_ragged_and_unequal_lengths(shape, causal, D, kernel_variant):
 
 
 # (B, H, Sq, Sk, D, causal): more work items than the chip has CUs, so that with attn.keep_on 2 (the default) a workgroup of
-# the four-wave 256-row kernel walks several of them and copies the next block's first tiles during a block's last ones
+# the 256-row kernel (both forms) walks several of them and copies the next block's first tiles during a block's last ones
 # (key counts that are a multiple of 256) or falls back to waiting (the others); heads in and out of the XCD dealing
 # (multiples of 8 or not); a ragged last key tile; fewer key tiles than the three copied ahead; Sq above Sk when causal.
 WALKED = [(4, 40, 1024, 1024, 128, False), (4, 40, 1000, 1000, 128, True), (3, 37, 900, 700, 64, False), (5, 24, 1536, 100, 128, False),
@@ -231,14 +231,15 @@ WALKED = [(4, 40, 1024, 1024, 128, False), (4, 40, 1000, 1000, 128, True), (3, 3
 
 @pytest.mark.parametrize("shape", WALKED)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
-def test_work_items_walked_by_one_workgroup_per_cu(shape, dtype):
+@pytest.mark.parametrize("form", [_lib.FO_ATTN_KERNEL_ROWS256_W4, _lib.FO_ATTN_KERNEL_ROWS256_W8])
+def test_work_items_walked_by_one_workgroup_per_cu(shape, dtype, form):
     B, H, Sq, Sk, D, causal = shape
     q, k, v = _qkv(B, H, Sq, Sk, D, dtype, seed=Sq + Sk)
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
     got = {}
-    _lib.tune_set("attn.variant", _lib.FO_ATTN_KERNEL_ROWS256_W4)
+    _lib.tune_set("attn.variant", form)
     try:
-        assert _kernel_taken(qd, kd, vd, causal) == _lib.FO_ATTN_KERNEL_ROWS256_W4
+        assert _kernel_taken(qd, kd, vd, causal) == form
         for mode in (0, 1, 2, -1):
             _lib.tune_set("attn.keep_on", mode)
             # (the allocator hands the blocks freed last to the next request of their size: the outputs start as NaN, and
