@@ -54,6 +54,8 @@ struct AttnParams {
   int n_qblk;
   int heavy_first;                      // 128-row kernel, causal: heads per group in the order of an XCD's workgroups, 0 = head by head (see launch_one)
   int order_n;                          // 128-row kernel, causal: entries of order_tab in use, 0 = none
+  int id_limit;                         // 256-row kernel: work items [0, id_limit) only (0 = all): the rest goes to a launch of the 128-row form
+  int tail_base;                        // 128-row pipelined form, non-causal: > 0 = this launch takes the 256-row work items from tail_base on, two workgroups each
   int keep_on;                          // 256-row kernel without bias: non-zero = copy the next query block's first tiles during the last tiles of a block
   uint8_t order_tab[kOrderTab];         // position in an XCD's launch order -> rank of the workgroup (0 = heaviest) that runs there
   DropoutParams drop;                   // used by the kernels instantiated with dropout only
@@ -668,9 +670,18 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
   // block's Q. The next block then starts without waiting for memory.
   constexpr bool KEEP_ON = BM == kWideBM && !VBIAS;
   const int n_bh = prm.B * prm.H;
-  const int n_items = PAIRED ? wide_items(prm.n_qblk, true) : prm.n_qblk;
-  const int n_ids = n_items * n_bh;
+  // (the tail of a launch of the 256-row kernel, taken over by this 128-row form: the 256-row blocks are what is dealt out)
+  const bool tail_mode = BM != kWideBM && !CAUSAL && prm.tail_base > 0;
+  const int n_items = PAIRED ? wide_items(prm.n_qblk, true) : tail_mode ? (prm.n_qblk + 1) / 2 : prm.n_qblk;
+  const int n_ids = (BM == kWideBM && prm.id_limit > 0) ? min(n_items * n_bh, prm.id_limit) : n_items * n_bh;
   auto decode = [&](int id, int& bh_, int& item_) {
+    int half = 0;
+    if (tail_mode) {
+      // workgroups 2 i and 2 i + 1 (16 j + x and 16 j + 8 + x where heads are dealt to XCDs, so that both stay on the
+      // XCD of the item) take the two 128-row halves of 256-row item tail_base + i
+      if ((n_bh & 7) == 0) { half = (id >> 3) & 1; id = prm.tail_base + ((id >> 4) << 3) + (id & 7); }
+      else { half = id & 1; id = prm.tail_base + (id >> 1); }
+    }
     if ((n_bh & 7) == 0) {
       const int x = id & 7, j = id >> 3;          // XCD, position in that XCD's list
       if (BM != kWideBM && CAUSAL && prm.heavy_first > 0) {
@@ -689,10 +700,12 @@ __global__ void __launch_bounds__(BM / (32 * QB) * 64, (BM == kWideBM || D == 12
       item_ = id / n_bh;
     }
     if (BM != kWideBM && CAUSAL) item_ = prm.n_qblk - 1 - item_;   // heaviest first
+    if (tail_mode) item_ = 2 * item_ + half;
   };
   int wg_id = blockIdx.x;
   int bh, item;
   decode(wg_id, bh, item);
+  if (tail_mode && item * BM >= prm.Sq) return;        // (the second half of a last block that has only one)
   int pass = 0;
   bool first_block = true, prefetched = false;
   bool o_rows_whole = false;     // every row of the block before this one was stored (no store instruction may have been skipped)
@@ -1325,6 +1338,9 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
   if (VBIAS && (p.Sk + kBN - 1) / kBN * kBN > kVBiasKeys) return FO_ERR_UNSUPPORTED;
   p.n_qblk = (p.Sq + BM - 1) / BM;
   unsigned grid = (unsigned)((BM == kWideBM ? wide_items(p.n_qblk, CAUSAL) : p.n_qblk) * p.B * p.H);
+  if (BM == kWideBM) { p.tail_base = 0; if (p.id_limit > 0 && grid > (unsigned)p.id_limit) grid = (unsigned)p.id_limit; }
+  else { p.id_limit = 0; if (CAUSAL) p.tail_base = 0; }
+  if (BM != kWideBM && p.tail_base > 0) grid = 2u * (unsigned)(wide_items((p.Sq + kWideBM - 1) / kWideBM, false) * p.B * p.H - p.tail_base);
   p.keep_on = 0;
   if (KEEP_ON) {
     // attn.keep_on: 0 = one work item per workgroup and no copies ahead for the next query block; 1 = copies ahead for
@@ -1343,6 +1359,30 @@ static int launch_wide(AttnParams p, hipStream_t stream) {
   if (attr != hipSuccess) return FO_ERR_LAUNCH;
   attn_fwd_wide_kernel<T, D, CAUSAL, QB, DBG, BM, VBIAS><<<grid, BM / (32 * QB) * 64, lds, stream>>>(p);
   return launch_status();
+}
+
+// The four-wave 256-row kernel, non-causal, whose last round of one workgroup per CU would be half empty or emptier:
+// the work items of that round go to a second launch, of the 128-row pipelined form, two workgroups per item. A 128-row
+// workgroup takes about two thirds of the time of a 256-row one, and that round is paid at that price instead of in
+// full. Measured (the chip holds a power budget, so a round in which only half the CUs work is already cheaper than a full
+// one): 12 heads x 8192 keys, 384 items on 256 CUs, 381 -> 363 us; 12 x 6144, 288 items, 290 -> 256; 33 x 4096, 528 items,
+// 315 -> 295; 36 x 2048 108 -> 101; 4 x 40 heads x 1024 keys 96-98 -> 98: from 2048 keys on. (attn.tail 0 switches it off.)
+template <typename T, int D, bool VBIAS>
+static int launch_rows256_w4_noncausal(AttnParams p, hipStream_t stream) {
+  p.id_limit = 0;
+  p.tail_base = 0;
+  const int n_cu = device_cus();
+  const int64_t ids = (int64_t)((p.Sq + kWideBM - 1) / kWideBM) * p.B * p.H;
+  const int64_t tail = ids % n_cu;
+  if (D == 128 && tune(g_attn_tail) != 0 && (n_cu & 7) == 0 && ids > n_cu && tail > 0 && 2 * tail <= n_cu && p.Sk >= 2048) {
+    AttnParams head = p, rest = p;
+    head.id_limit = (int)(ids - tail);
+    rest.tail_base = (int)(ids - tail);
+    const int rc = launch_wide<T, D, false, 2, 0, kWideBM, VBIAS>(head, stream);
+    if (rc != FO_OK) return rc;
+    return launch_wide<T, D, false, 1, 0, kBM, VBIAS>(rest, stream);
+  }
+  return launch_wide<T, D, false, 2, 0, kWideBM, VBIAS>(p, stream);
 }
 
 template <typename T, int D, bool CAUSAL, bool LAZY, int DBG, bool DROP = false, bool BIAS = false, bool KBIAS = false>
@@ -1424,7 +1464,16 @@ static int choose_kernel(const AttnParams& p, int D, bool causal, bool dropout, 
     // With the rounds filled to less than 80 % the 128-row kernel (two workgroups per CU, finer blocks, heaviest first)
     // was 1-5 % faster (B*H = 160-192 at 512-1024 keys, 48 heads x 4096 causal), from 83 % on the 256-row kernel 3-6 %.
     const int64_t rounds = (wide_wgs + n_cu - 1) / n_cu;
-    bool wide = wide_ok && wide_wgs >= n_cu && wide_wgs * 10 >= rounds * n_cu * (D == 128 && keys >= 4096 ? 7 : 8);
+    // (non-causal at head_dim 128 a last round that is at most half full goes to a second launch of the 128-row form,
+    // launch_rows256_w4_noncausal, and counts 0.6 of a round: 33 heads x 4096 keys, 528 items, 295 us that way against
+    // 359 us on the 128-row kernel; 12 heads x 6144 keys, 288 items, 256 against 288 us)
+    int64_t tenths = rounds * 10;
+    {
+      const int64_t tail = wide_wgs % n_cu;
+      if (!causal && D == 128 && p.Sk >= 2048 && tune(g_attn_tail) != 0 && (n_cu & 7) == 0 && wide_wgs > n_cu && tail > 0 && 2 * tail <= n_cu)
+        tenths = (rounds - 1) * 10 + 6;
+    }
+    bool wide = wide_ok && wide_wgs >= n_cu && wide_wgs * 100 >= tenths * n_cu * (D == 128 && keys >= 4096 ? 7 : 8);
     // (long rows of keys at head_dim 128: also with the rounds filled to 70-80 % - 12 heads x 8192 non-causal, 384
     // workgroups, 375 against 399 us - and with three quarters of a single round - 12 heads x 8192 causal 196 against 215 us,
     // 12 heads x 4096 non-causal 98 against 121 us)
@@ -1486,7 +1535,7 @@ int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
         if (v == FO_ATTN_KERNEL_ROWS128_PIPE)
           return causal ? launch_wide<T, D, true, 1, 0, kBM, true>(p, stream) : launch_wide<T, D, false, 1, 0, kBM, true>(p, stream);
         if (v == FO_ATTN_KERNEL_ROWS256_W4)
-          return causal ? launch_wide<T, D, true, 2, 0, kWideBM, true>(p, stream) : launch_wide<T, D, false, 2, 0, kWideBM, true>(p, stream);
+          return causal ? launch_wide<T, D, true, 2, 0, kWideBM, true>(p, stream) : launch_rows256_w4_noncausal<T, D, true>(p, stream);
         return causal ? launch_one<T, D, true, true, 0, false, false, true>(p, stream) : launch_one<T, D, false, true, 0, false, false, true>(p, stream);
       }
       return causal ? launch_one<T, D, true, true, 0, true, false, true>(p, stream) : launch_one<T, D, false, true, 0, true, false, true>(p, stream);
@@ -1498,7 +1547,7 @@ int launch(const AttnParams& p, bool causal, bool dropout, hipStream_t stream) {
   const int v = choose_kernel(p, D, causal, dropout, tune(g_attn_variant));
   if (v == FO_ATTN_KERNEL_ROWS256_W8) return causal ? launch_wide<T, D, true, 1>(p, stream) : launch_wide<T, D, false, 1>(p, stream);
   if (v == FO_ATTN_KERNEL_ROWS128_PIPE) return causal ? launch_wide<T, D, true, 1, 0, kBM>(p, stream) : launch_wide<T, D, false, 1, 0, kBM>(p, stream);
-  if (v == FO_ATTN_KERNEL_ROWS256_W4) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_wide<T, D, false, 2>(p, stream);
+  if (v == FO_ATTN_KERNEL_ROWS256_W4) return causal ? launch_wide<T, D, true, 2>(p, stream) : launch_rows256_w4_noncausal<T, D, false>(p, stream);
 #if defined(FO_ABLATIONS)
   // Timing ablations (WRONG results by design; bf16, head_dim 128 only). 256-row kernel, non-causal: 256 + bits for eight
   // waves, 512 + bits for four; bit 0 no global->LDS copies, 1 no exponentials, 2 no LDS fragment reads, 5 no wait for
@@ -1627,6 +1676,7 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
   for (int i = 0; i < 3; ++i) { p.qs[i] = qs[i]; p.ks[i] = ks[i]; p.vs[i] = vs[i]; p.os[i] = os[i]; }
   p.scale_log2e = softmax_scale * 1.4426950408889634f;
   p.n_qblk = (int)n_qblk;
+  p.heavy_first = 0; p.order_n = 0; p.id_limit = 0; p.tail_base = 0; p.keep_on = 0;
   const bool drop = dropout_p > 0.0f;
   p.drop = make_dropout(dropout_p, seed, rng_offset);
   p.bias.ptr = bias;

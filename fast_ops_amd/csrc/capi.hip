@@ -9,6 +9,7 @@ std::atomic<int> g_attn_variant{-1};
 std::atomic<int> g_attn_bwd_variant{-1};
 std::atomic<int> g_attn_order{-1};
 std::atomic<int> g_attn_keep_on{-1};
+std::atomic<int> g_attn_tail{-1};
 std::atomic<int> g_attn_balance{-1};
 std::atomic<int> g_attn_bwd_order{-1};
 }  // namespace fo
@@ -58,6 +59,10 @@ extern "C" int fo_tune_set(const char* key, int value) {
     if (value > 2) return FO_ERR_UNSUPPORTED;
     fo::g_attn_keep_on = value; return FO_OK;
   }
+  if (strcmp(key, "attn.tail") == 0) {
+    if (value > 1) return FO_ERR_UNSUPPORTED;                         // 0 = one launch, 1 = a half-empty last round goes to the 128-row form (default)
+    fo::g_attn_tail = value; return FO_OK;
+  }
   if (strcmp(key, "attn.balance") == 0) {
     if (value > 1) return FO_ERR_UNSUPPORTED;                         // 0 = plain order, 1 = balanced where it applies (default)
     fo::g_attn_balance = value; return FO_OK;
@@ -73,6 +78,7 @@ extern "C" int fo_tune_get(const char* key) {
   if (strcmp(key, "attn_bwd.variant") == 0) return fo::tune(fo::g_attn_bwd_variant);
   if (strcmp(key, "attn.order") == 0) return fo::tune(fo::g_attn_order);
   if (strcmp(key, "attn.keep_on") == 0) return fo::tune(fo::g_attn_keep_on);
+  if (strcmp(key, "attn.tail") == 0) return fo::tune(fo::g_attn_tail);
   if (strcmp(key, "attn.balance") == 0) return fo::tune(fo::g_attn_balance);
   if (strcmp(key, "attn_bwd.order") == 0) return fo::tune(fo::g_attn_bwd_order);
   if (strcmp(key, "build.ablations") == 0) {

@@ -27,6 +27,7 @@ extern std::atomic<int> g_attn_variant;
 extern std::atomic<int> g_attn_bwd_variant;
 extern std::atomic<int> g_attn_bwd_order;   // attention backward: -1 automatic, 0 all heads in one group, n > 0 groups of n heads
 extern std::atomic<int> g_attn_balance;   // 128-row attention kernel, causal: 0 plain heaviest-first order also where a launch fits the chip at once, otherwise (default) balanced
+extern std::atomic<int> g_attn_tail;      // 256-row attention kernel, non-causal: 0 = never hand the last round to the 128-row form (see launch_rows256_w4_noncausal)
 extern std::atomic<int> g_attn_keep_on;   // 256-row attention kernel, four waves: see launch_wide
 extern std::atomic<int> g_attn_order;   // 128-row attention kernel, causal: -1 automatic, 0 head by head, n > 0 heaviest query blocks first within groups of n heads per XCD
 inline int tune(const std::atomic<int>& v) { return v.load(std::memory_order_relaxed); }

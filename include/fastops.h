@@ -46,7 +46,7 @@ const char* fo_strerror(int status);
 int fo_version(void);
 
 /* Tuning hook for benchmarks, profiling and tests: selects a kernel variant or a workgroup order by name
- * ("lion.variant", "attn.variant", "attn_bwd.variant", "attn.order", "attn.balance", "attn.keep_on", "attn_bwd.order"). Every value it accepts selects
+ * ("lion.variant", "attn.variant", "attn_bwd.variant", "attn.order", "attn.balance", "attn.keep_on", "attn.tail", "attn_bwd.order"). Every value it accepts selects
  * code that computes the same function as the default; value -1 restores the default (the measured best). Returns
  * FO_OK, or FO_ERR_UNSUPPORTED for an unknown key or a value that selects nothing. The settings are process-global
  * atomics: a call reads each one once, a call already issued is not affected. fo_tune_get additionally answers

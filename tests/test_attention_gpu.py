@@ -263,6 +263,51 @@ def test_work_items_walked_by_one_workgroup_per_cu(shape, dtype, form):
         _check(o[b:b + 1, h:h + 1], lse[b:b + 1, h:h + 1], o_ref, lse_ref, f"{shape} {dtype} slice ({b},{h})")
 
 
+# (B, H, Sq, Sk): non-causal head_dim 128 shapes whose 256-row work items fill one or more rounds of one workgroup per CU
+# and leave a last round that is at most half full (on 256 CUs: 384 = 256 + 128, 640 = 512 + 128, 264 = 256 + 8, and 330
+# with heads that are not dealt to XCDs and a last block of 44 rows, whose second 128-row half does not exist): the items
+# of that round go to a second launch of the 128-row pipelined form (attn.tail, default on).
+TAILS = [(1, 12, 8192, 2048), (4, 40, 1024, 2100), (1, 8, 8448, 2048), (2, 15, 2604, 2500)]
+
+
+@pytest.mark.parametrize("shape", TAILS)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_last_round_handed_to_the_128_row_form(shape, dtype, with_bias):
+    from fast_ops_amd.flash_attention.flash_attention import attn_fwd_strided
+
+    B, H, Sq, Sk = shape
+    D = 128
+    q, k, v = _qkv(B, H, Sq, Sk, D, dtype, seed=Sq)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    bias = None
+    if with_bias:
+        bias = torch.randn(B, 1, 1, Sk, generator=torch.Generator().manual_seed(Sk)).to(dtype)   # one value per key
+    got = {}
+    _lib.tune_set("attn.variant", _lib.FO_ATTN_KERNEL_ROWS256_W4)
+    try:
+        assert _kernel_taken(qd, kd, vd, False) == _lib.FO_ATTN_KERNEL_ROWS256_W4
+        for mode in (0, 1):
+            _lib.tune_set("attn.tail", mode)
+            junk = (torch.full_like(qd, float("nan")), torch.full((B, H, Sq), float("nan"), device=DEV))   # (see the test above)
+            del junk
+            o, lse = attn_fwd_strided(qd, kd, vd, (0, 1, 2, 3), False, None, None, None if bias is None else bias.to(DEV))
+            torch.cuda.synchronize()
+            got[mode] = (o.cpu(), lse.cpu())
+            assert torch.isfinite(got[mode][0].float()).all() and torch.isfinite(got[mode][1]).all(), f"attn.tail {mode}"
+    finally:
+        _lib.tune_set("attn.tail", -1)
+        _lib.tune_set("attn.variant", -1)
+    # two forms of one pipeline: the same scores and sums, P rounded against references that may differ
+    assert float((got[0][1] - got[1][1]).abs().max()) <= 1e-4
+    assert float(((got[0][0].float() - got[1][0].float()).abs() - (2e-2 + 2e-2 * got[0][0].float().abs())).max()) <= 0
+    o, lse = got[1]
+    for b, h in [(0, 0), (B - 1, H - 1), (B - 1, H // 2)]:          # the last heads are the ones in the last round
+        o_ref, lse_ref = attention_fwd_oracle(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1],
+                                              bias=None if bias is None else bias[b:b + 1])
+        _check(o[b:b + 1, h:h + 1], lse[b:b + 1, h:h + 1], o_ref, lse_ref, f"{shape} {dtype} bias={with_bias} slice ({b},{h})")
+
+
 @pytest.mark.parametrize("shape", [(1, 2, 600, 700), (1, 1, 513, 1025), (2, 2, 255, 64), (1, 1, 770, 770)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)

@@ -151,7 +151,7 @@ def test_tune_hook():
     assert lib.fo_tune_set(b"lion.variant", -1) == 0
     assert lib.fo_tune_set(b"no.such.key", 1) == -8
     # every key the kernels read: default -1 (the library's choice), settable, readable
-    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn.balance", 0), (b"attn.keep_on", 1), (b"attn_bwd.order", 2)):
+    for key, value in ((b"attn.variant", 16), (b"attn_bwd.variant", 0), (b"attn.order", 2), (b"attn.balance", 0), (b"attn.keep_on", 1), (b"attn.tail", 0), (b"attn_bwd.order", 2)):
         assert lib.fo_tune_get(key) == -1
         assert lib.fo_tune_set(key, value) == 0 and lib.fo_tune_get(key) == value
         assert lib.fo_tune_set(key, -1) == 0 and lib.fo_tune_get(key) == -1
@@ -211,6 +211,10 @@ def test_attn_kernel_query_and_stride_limit_without_device_work():
         assert k(32, 16, 512, 512, 128, 1) == R128           # causal below 1024 queries
         assert k(16, 16, 512, 512, 128, 0) == W4 and k(10, 16, 512, 512, 128, 0) == R128   # 512 / 320 workgroups; non-causal: four waves
         assert k(32, 16, 256, 256, 128, 0) == W8             # (below 512 keys the eight-wave form stays)
+        # a last round that is at most half full goes to a second launch of the 128-row form and counts 0.6 of a round:
+        # 528 items = 2 rounds + 16, 288 = 1 round + 32 (from 4096 keys on the rounds need to be filled to 70 %); not causal
+        assert k(1, 33, 4096, 4096, 128, 0) == W4 and k(1, 12, 6144, 6144, 128, 0) == W4 and k(1, 33, 4096, 4096, 128, 1) != W4
+        assert k(1, 36, 2048, 2048, 128, 0) == R128          # 288 items, but below 4096 keys the bar is 80 %
         assert k(1, 8, 8192, 8192, 64, 0) == W4 and k(4, 8, 4096, 4096, 64, 0) == W4 and k(8, 8, 2048, 2048, 64, 0) == R128   # head_dim 64: long rows only,
         assert k(1, 8, 16384, 16384, 64, 1) == W4 and k(2, 16, 8192, 8192, 64, 1) == W4 and k(4, 16, 4096, 4096, 64, 1) == W4  # and four waves
         assert k(8, 16, 2048, 2048, 64, 1) == R128 and k(4, 16, 4096, 4096, 64, 1, bias=2) == R128   # (causal from 4096 keys, with a per-key bias from 8192)
