@@ -11,7 +11,9 @@ other three benchmark configurations ("configs": GPT-2-small attention forward, 
 attention forward at B=16 H=32 S=2048 D=128), and the rate of the vendor library's plain bf16 GEMM on random operands
 on the same box ("library_gemm": what MFMA code reaches here at all), and three variations of the headline launch
 ("headline_variants": the same shape non-causal, the same causal launch on all-zero operands, and head_dim 64 at
-B=2 H=32 S=8192 causal) with the ratio of the causal time to half the non-causal time.
+B=2 H=32 S=8192 causal) with the ratio of the causal time to half the non-causal time, and the headline launch and the
+B=16 H=32 S=2048 launch once more with one work item per workgroup (attn.keep_on 0) instead of workgroups that walk
+their share of the items.
 
 `--path next` times what lies around the two headline kernels with the same machinery: attention forward, backward and
 forward+backward on the reference's own benchmark matrix (1 x 12 heads x {2048, 4096, 8192} x 128, bf16, with and
@@ -322,6 +324,16 @@ def bench_attention(steps, warmup, settle, cpu_baseline, extras):
             "head_dim_64": _attn_rate(2, 32, 8192, 64, torch.bfloat16, True, steps, warmup, settle),
         }
         hv["causal_over_half_noncausal"] = hv["causal"]["kernel_ms_avg"] / (0.5 * hv["noncausal"]["kernel_ms_avg"])
+        # what the workgroups' walk over the work items is worth (attn.keep_on 0: one item per workgroup, no copies ahead
+        # for the next query block), at the headline shape and at B=16 H=32 S=2048 fp16 non-causal, whose query blocks are short
+        from fast_ops_amd import _lib
+
+        _lib.tune_set("attn.keep_on", 0)
+        try:
+            hv["causal_one_item_per_workgroup"] = _attn_rate(B, H, S, D, torch.bfloat16, True, steps, warmup, settle)
+            hv["config_5a_one_item_per_workgroup"] = _attn_rate(16, 32, 2048, 128, torch.float16, False, steps, warmup, settle)
+        finally:
+            _lib.tune_set("attn.keep_on", -1)
         res["headline_variants"] = hv
         torch.cuda.empty_cache()
         # the other attention configurations: report only

@@ -60,6 +60,7 @@ def test_default_run_prints_one_json_line_with_the_agreed_keys():
     assert set(d["configs"]) >= {"2_attn_fwd_gpt2_small", "3_lion_gpt2_small", "5a_attn_fwd_throughput"}
     # the headline launch varied one thing at a time (mask, operand bits, head_dim), and the ratio the causal form pays
     hv = d["headline_variants"]
-    assert set(hv) >= {"causal", "noncausal", "zero_operands", "zero_operands_noncausal", "head_dim_64", "causal_over_half_noncausal"}
+    assert set(hv) >= {"causal", "noncausal", "zero_operands", "zero_operands_noncausal", "head_dim_64", "causal_over_half_noncausal", "causal_one_item_per_workgroup",
+                       "config_5a_one_item_per_workgroup"}
     assert hv["causal_over_half_noncausal"] == pytest.approx(hv["causal"]["kernel_ms_avg"] / (0.5 * hv["noncausal"]["kernel_ms_avg"]), rel=1e-9)
     assert "bwd" in d["configs"]["2_attn_fwd_gpt2_small"] and "training_loop" in d["configs"]["3_lion_gpt2_small"]
